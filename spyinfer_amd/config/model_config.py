@@ -405,3 +405,123 @@ class SodedraConfig(ModelConfig):
                 if E <= 0 or G <= 0 or E % G or not 0 < f["keep"] <= G or not 0 < f["top"] <= f["keep"] * (E // G):
                     raise ConfigError("%s.mlp.router: %d choices among %d of %d groups of %d experts cannot be made"
                                       % (where, f["top"], f["keep"], G, E))
+
+
+@dataclasses.dataclass
+class MeronexConfig(ModelConfig):
+    """Meronex: pre-norm layers whose sublayers' results are multiplied by a sigmoid gate of the sublayer's input and by a
+    constant before they meet the stream; norms over consecutive groups of the vector; token mixers 'mlstm' (a matrix
+    memory with exponential gates), 'delta' (a gated delta rule with short convolutions and one decay per head) and
+    'parallel' (an attention with rescaled rotation, normed values and capped scores beside a time mix with token shift
+    and a decay per key channel, their normed results averaged); feed-forwards 'moe' (experts with a clamped activation
+    whose sigmoid scores multiply the experts' input) or none.  The configuration is nested; ``layers`` lists every
+    layer's type and sizes, and nothing is assumed equal between layers."""
+
+    architecture: str = ""
+    vocab: int = -1
+    width: int = -1
+    norm_eps: float = 0.0
+    norm_groups: int = 1
+    residual_mult: float = 1.0
+    #: one dict per layer: type, mixer (sizes and constants of that mixer), mlp (None or {kind: moe, ff, limit, experts, top})
+    layers: List[Dict[str, Any]] = dataclasses.field(default_factory=list)
+
+    MIXERS: ClassVar[tuple] = ("mlstm", "delta", "parallel")
+
+    @classmethod
+    def from_dict(cls, raw: Dict[str, Any]) -> "MeronexConfig":
+        cfg = cls(architecture=str(raw.get("architecture") or (raw.get("architectures") or [""])[0]),
+                  vocab=_need(raw, "vocab", int), width=_need(raw, "width", int), norm_eps=float(_need(raw, "norm.eps", (int, float))))
+        if (raw.get("norm") or {}).get("groups") is not None:
+            cfg.norm_groups = _need(raw, "norm.groups", int)
+        if raw.get("residual_mult") is not None:
+            cfg.residual_mult = float(_need(raw, "residual_mult", (int, float)))
+        cfg.layers = [cls._layer(i, l) for i, l in enumerate(_need(raw, "layers", list))]
+        cfg._raw = dict(raw)
+        cfg.validate()
+        return cfg
+
+    @staticmethod
+    def _attention(m: Dict[str, Any], at: str) -> Dict[str, Any]:
+        mix = {k: _need(m, k, int, at) for k in ("heads", "dim", "vdim")}
+        mix["kv_heads"] = _need(m, "kv_heads", int, at) if m.get("kv_heads") is not None else mix["heads"]
+        mix["scale"] = float(_need(m, "scale", (int, float), at))
+        mix["softcap"] = float(_need(m, "softcap", (int, float), at)) if m.get("softcap") is not None else 0.0
+        rot = m.get("rot")
+        mix["rot"] = None
+        if rot:
+            mix["rot"] = {"base": float(_need(rot, "base", (int, float), at + ".rot")), "dims": _need(rot, "dims", int, at + ".rot"),
+                          "scaling": None}
+            sc = rot.get("scaling")
+            if sc:
+                mix["rot"]["scaling"] = {k: float(_need(sc, k, (int, float), at + ".rot.scaling")) for k in ("factor", "original", "fast", "slow")}
+        return mix
+
+    @classmethod
+    def _layer(cls, i: int, raw: Dict[str, Any]) -> Dict[str, Any]:
+        where = "config.json layers[%d]" % i
+        if not isinstance(raw, dict):
+            raise ConfigError("%s is no object" % where)
+        kind = _need(raw, "type", str, where)
+        if kind not in cls.MIXERS:
+            raise ConfigError("%s: mixer type %r is not known (%s)" % (where, kind, ", ".join(cls.MIXERS)))
+        m = _need(raw, "mixer", dict, where)
+        at = where + ".mixer"
+        if kind == "mlstm":
+            mix = {k: _need(m, k, int, at) for k in ("heads", "dim", "vdim")}
+            mix["gate_cap"] = float(_need(m, "gate_cap", (int, float), at))
+        elif kind == "delta":
+            mix = {k: _need(m, k, int, at) for k in ("heads", "dim", "vdim", "conv")}
+            mix["kv_heads"] = _need(m, "kv_heads", int, at) if m.get("kv_heads") is not None else mix["heads"]
+        else:
+            right = _need(m, "right", dict, at)
+            mix = {"left": cls._attention(_need(m, "left", dict, at), at + ".left"),
+                   "right": {k: _need(right, k, int, at + ".right") for k in ("heads", "dim")}}
+        out = {"type": kind, "mixer": mix, "mlp": None}
+        mlp = raw.get("mlp")
+        if mlp is not None:
+            at = where + ".mlp"
+            fk = _need(mlp, "kind", str, at)
+            if fk != "moe":
+                raise ConfigError("%s: kind %r is not known (moe)" % (at, fk))
+            out["mlp"] = {"kind": fk, "ff": _need(mlp, "expert.ff", int, at), "limit": float(_need(mlp, "expert.limit", (int, float), at)),
+                          "experts": _need(mlp, "router.experts", int, at), "top": _need(mlp, "router.top", int, at)}
+        return out
+
+    def to_dict(self) -> Dict[str, Any]:
+        return dict(getattr(self, "_raw", {}))
+
+    def validate(self) -> None:
+        if self.vocab <= 0 or self.width <= 0:
+            raise ConfigError("config.json: vocab and width must be positive")
+        if not (self.norm_eps > 0.0):
+            raise ConfigError("config.json: norm.eps must be positive")
+        if self.norm_groups <= 0 or self.width % self.norm_groups:
+            raise ConfigError("config.json: norm.groups (%d) must divide the width (%d)" % (self.norm_groups, self.width))
+        if not self.layers:
+            raise ConfigError("config.json: no layers")
+        for i, layer in enumerate(self.layers):
+            where = "config.json layers[%d]" % i
+            sides = [("", layer["mixer"])] if layer["type"] != "parallel" else [(".left", layer["mixer"]["left"]), (".right", layer["mixer"]["right"])]
+            for side, m in sides:
+                if any(isinstance(v, int) and not isinstance(v, bool) and v <= 0 for v in m.values()):
+                    raise ConfigError("%s.mixer%s: sizes must be positive" % (where, side))
+                if "kv_heads" in m and m["heads"] % m["kv_heads"]:
+                    raise ConfigError("%s.mixer%s: heads (%d) is not a multiple of kv_heads (%d)" % (where, side, m["heads"], m["kv_heads"]))
+            if layer["type"] == "mlstm" and not layer["mixer"]["gate_cap"] > 0.0:
+                raise ConfigError("%s.mixer.gate_cap must be positive" % where)
+            if layer["type"] == "delta" and layer["mixer"]["conv"] > 8:
+                raise ConfigError("%s.mixer.conv: at most 8 taps" % where)
+            if layer["type"] == "parallel":
+                left = layer["mixer"]["left"]
+                if left["softcap"] < 0.0:
+                    raise ConfigError("%s.mixer.left.softcap must not be negative" % where)
+                rot = left["rot"]
+                if rot and (rot["dims"] % 2 or not (0 < rot["dims"] <= left["dim"]) or not rot["base"] > 1.0):
+                    raise ConfigError("%s.mixer.left.rot: dims must be even and at most dim, base above 1" % where)
+                sc = rot["scaling"] if rot else None
+                if sc and not (sc["factor"] > 0.0 and sc["original"] > 0.0 and sc["fast"] > 0.0 and sc["slow"] > 0.0):
+                    raise ConfigError("%s.mixer.left.rot.scaling: factor, original, fast and slow must be positive" % where)
+            f = layer["mlp"]
+            if f and (f["ff"] <= 0 or not f["limit"] > 0.0 or f["experts"] <= 0 or not 0 < f["top"] <= f["experts"]):
+                raise ConfigError("%s.mlp: inner size and limit positive, 1 to %d choices" % (where, max(f["experts"], 1)))

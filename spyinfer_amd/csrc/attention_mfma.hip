@@ -132,10 +132,11 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, bf16_t* kc, bf16_t* vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
-    int n_q, int n_kv, int d, float scale, int window, int splits, float* __restrict__ ws, FusedQKV fz, int out_tiles,
+    int n_q, int n_kv, int d, float scale, int window, float softcap, int splits, float* __restrict__ ws, FusedQKV fz, int out_tiles,
     unsigned* counters, int log2p, const int* __restrict__ pieces) {
     constexpr int KK = DMAX / 32;   // 32-wide chunks of the head dim for Q.K
     constexpr int DT = DMAX / 16;   // 16-row tiles of the head dim for P.V
+    const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
     extern __shared__ float lds[];   // the waves' O, m, l: AW (head sizes up to 128) or AW - 1 times (DT * 4 + 2) * 64 floats
     // Which (tile, kv head, part of the keys) this block has: its place in the grid, or (FUSED, `pieces` given) a record
     // of 8 ints that the host made for this block: { entry, kv head, first and end block of 32 keys, number of this
@@ -393,7 +394,8 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int key = c0 + 8 * g + j;
-            const float v = (j < 4 ? sa[j] : sb[j - 4]) * scale;
+            float v = (j < 4 ? sa[j] : sb[j - 4]) * scale;
+            if (softcap > 0.f) v = softcap * capped_tanh(v * inv_cap);          // scores capped: cap tanh(score / cap)
             const bool ok = row_ok && key <= pos && key >= lo_row && key < kvl;
             sc[j] = ok ? v : -INFINITY;
             bmax = fmaxf(bmax, sc[j]);
@@ -653,7 +655,7 @@ extern "C" int64_t spy_attention_mfma_workspace(int num_tiles, int n_kv, int d, 
 extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, int P, int num_pages, const int* cu_q,
                                   const int* pos0, const int* kv_len, const int* block_table, int max_blocks, const int* tile_entry,
                                   const int* tile_row0, int num_tiles, int S, int T, int n_q, int n_kv, int d, float scale,
-                                  int window, int splits, float* ws, const void* qkv, const void* qw, const void* kw, int w_dtype,
+                                  int window, float softcap, int splits, float* ws, const void* qkv, const void* qw, const void* kw, int w_dtype,
                                   float eps, const float* cos_t, const float* sin_t, int max_pos, int store, int out_tiles,
                                   unsigned* counters, int n_counters, const int* pieces, int num_pieces, hipStream_t st) {
     SPY_REQUIRE(num_tiles > 0 && S > 0 && T > 0 && n_q > 0 && n_kv > 0 && num_pages > 0 && max_blocks > 0,
@@ -666,6 +668,7 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
     SPY_REQUIRE(n_kv <= 65535, "spy_attention_mfma: too many kv heads");
     SPY_REQUIRE(out_tiles >= 0 && out_tiles <= 8 && (!out_tiles || (T <= 16 * out_tiles && (n_q * d) % 32 == 0 && d % 8 == 0)),
                 "spy_attention_mfma: operand order is for at most 128 rows (%d here) of a width that is a multiple of 32", T);
+    SPY_REQUIRE(softcap >= 0.f && (!qkv || softcap == 0.f), "spy_attention_mfma: the scores' cap must not be negative, and the fused variant takes none");
     FusedQKV fz = {(const bf16_t*)qkv, qw, kw, w_dtype, eps, cos_t, sin_t, max_pos, store};
     if (qkv) {
         SPY_REQUIRE(T == S && num_tiles == S, "spy_attention_mfma: the fused variant takes single tokens only (%d tokens of %d entries)", T, S);
@@ -695,7 +698,7 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
 #define ATT_LAUNCH(DM, FZ, FL)                                                                                                \
     attention_mfma_kernel<DM, FZ, FL><<<grid, AW * 64, (DM <= 128 ? AW : AW - 1) * ((DM / 16) * 4 + 2) * 64 * sizeof(float), st>>>(  \
         (bf16_t*)out, (const bf16_t*)q, (bf16_t*)kc, (bf16_t*)vc, P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,  \
-        tile_entry, tile_row0, n_q, n_kv, d, scale, window, splits, ws, fz, out_tiles, cnt, log2p, pieces)
+        tile_entry, tile_row0, n_q, n_kv, d, scale, window, softcap, splits, ws, fz, out_tiles, cnt, log2p, pieces)
 #define ATT_CASE(DM)                                                                                                          \
     if (qkv && P <= 32) ATT_LAUNCH(DM, true, FULL_STREAMED); else if (qkv) ATT_LAUNCH(DM, true, FULL_KEPT);                      \
     else if (d == DM && P <= 32) ATT_LAUNCH(DM, false, FULL_STREAMED); else if (d == DM) ATT_LAUNCH(DM, false, FULL_KEPT);       \

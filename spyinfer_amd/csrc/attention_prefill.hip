@@ -37,7 +37,7 @@ __global__ __launch_bounds__(PF_ROWS / RT * 4, MINW) void attention_prefill_kern
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
-    int n_q, int n_kv, int d, float scale, int window, int log2p, int num_tiles, int splits, float* __restrict__ ws, int out_tiles) {
+    int n_q, int n_kv, int d, float scale, int window, float softcap, int log2p, int num_tiles, int splits, float* __restrict__ ws, int out_tiles) {
     constexpr int KK = DMAX / 32, DT = DMAX / 16;
     // 16 elements of padding per staged row: the products' 16-byte reads then have no bank conflicts (measured with
     // SQ_LDS_BANK_CONFLICT: 40 % of the LDS cycles with 8, none with 16; the kernel's time follows only by 0-3 %)
@@ -118,6 +118,7 @@ __global__ __launch_bounds__(PF_ROWS / RT * 4, MINW) void attention_prefill_kern
     const bool w_rows_full = w_first_row + 16 * RT - 1 < nrows;                             // all rows of the wave exist
     const int w_min_pos = p0 + w_first_row / G;                                            // keys up to here are before every row
     const int w_max_lo = window > 0 ? max(0, w_hi - window + 1) : 0;                       // keys from here on are in every window
+    const float cap_over_scale = softcap > 0.f ? softcap / scale : 0.f, scale_over_cap = softcap > 0.f ? scale / softcap : 0.f;
     const float scale2 = scale * 1.4426950408889634f;                                      // scores times log2(e)
 
     f32x4_t acc[RT][DT];
@@ -248,6 +249,11 @@ __global__ __launch_bounds__(PF_ROWS / RT * 4, MINW) void attention_prefill_kern
                 float sc[8];                          // raw scores; the scale goes into the exponent's fma
 #pragma unroll
                 for (int j = 0; j < 8; ++j) sc[j] = j < 4 ? sa[t][j] : sb[t][j - 4];
+                if (softcap > 0.f) {
+                    // capped scores, cap tanh(score scale / cap), kept over the scale so that what follows is as without a cap
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) sc[j] = cap_over_scale * capped_tanh(sc[j] * scale_over_cap);
+                }
                 if (!unmasked) {
                     // (the empty statement keeps the masks' index arithmetic inside this branch: the compiler had moved
                     // it ahead of the branch, into the path of every block of keys)
@@ -383,7 +389,7 @@ static long long cu_count() {
 extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, const void* vc, int P, int num_pages, const int* cu_q,
                                      const int* pos0, const int* kv_len, const int* block_table, int max_blocks,
                                      const int* tile_entry, const int* tile_row0, int num_tiles, int tile_rows, int S, int T, int n_q,
-                                     int n_kv, int d, float scale, int window, int splits, float* ws, int out_tiles, hipStream_t st) {
+                                     int n_kv, int d, float scale, int window, float softcap, int splits, float* ws, int out_tiles, hipStream_t st) {
     SPY_REQUIRE(num_tiles > 0 && S > 0 && T > 0 && n_q > 0 && n_kv > 0 && num_pages > 0 && max_blocks > 0,
                 "spy_attention_prefill: empty operand");
     SPY_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "spy_attention_prefill: head_dim %d is not a multiple of 16 in 16..128", d);
@@ -404,7 +410,7 @@ extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, c
     const dim3 mgrid(num_tiles * (tile_rows / 16), n_kv);
     const bool one_per_cu = (long long)grid.x * grid.y * grid.z <= cu_count();
 #define PF_ARGS (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, P, num_pages, cu_q, pos0, kv_len, block_table,   \
-                max_blocks, tile_entry, tile_row0, n_q, n_kv, d, scale, window, log2p, num_tiles, splits, ws, out_tiles
+                max_blocks, tile_entry, tile_row0, n_q, n_kv, d, scale, window, softcap, log2p, num_tiles, splits, ws, out_tiles
     // (head sizes other than 64 and 128 keep the 4-wave shape: with conditions in the head-dim loops the other needs too many registers)
 #define PF_CASE(DM)                                                                                                              \
     if (tile_rows == 256) attention_prefill_kernel<DM, true, 2, 2, 256><<<grid, 512, 0, st>>>(PF_ARGS);                          \

@@ -130,21 +130,25 @@ template <> struct Vec4<bf16_t> {
 template <typename TA, typename TW, bool VEC>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restrict__ delta, const TA* __restrict__ delta2,
                                    const TW* __restrict__ w, float eps, TA* __restrict__ out, const int* __restrict__ rows, int T,
-                                   int H) {
+                                   int H, int ld) {
+    // H: values that are normed together: the whole row (ld == H), or one of the row's ld / H consecutive groups, which
+    // blockIdx.y counts
     __shared__ float red[16];
     const int r = blockIdx.x;
+    const size_t g0 = (size_t)blockIdx.y * H;
     int t = r;
     if (rows) {
         t = rows[r];
         if (t < 0 || t >= T) {   // never the case for a checked batch; write zeros rather than read outside
-            for (int i = threadIdx.x; i < H; i += blockDim.x) out[(size_t)r * H + i] = from_f32<TA>(0.f);
+            for (int i = threadIdx.x; i < H; i += blockDim.x) out[(size_t)r * ld + g0 + i] = from_f32<TA>(0.f);
             return;
         }
     }
-    float* x = resid + (size_t)t * H;
-    const TA* dl = delta ? delta + (size_t)t * H : nullptr;
-    const TA* dl2 = delta2 ? delta2 + (size_t)t * H : nullptr;
-    TA* o = out + (size_t)r * H;
+    float* x = resid + (size_t)t * ld + g0;
+    const TA* dl = delta ? delta + (size_t)t * ld + g0 : nullptr;
+    const TA* dl2 = delta2 ? delta2 + (size_t)t * ld + g0 : nullptr;
+    TA* o = out + (size_t)r * ld + g0;
+    w += g0;
     const bool write_back = dl && !rows;
     if (VEC) {
         // H % 4 == 0 and 16-byte aligned rows (checked by the launcher); the row fits the register passes
@@ -204,19 +208,22 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
 }
 
 extern "C" int spy_add_rmsnorm(float* resid, const void* delta, const void* delta2, const void* w, int w_dtype, float eps, void* out,
-                               int out_dtype, const int* rows, int n_out, int T, int H, hipStream_t st) {
-    SPY_REQUIRE(n_out > 0 && T > 0 && H > 0, "spy_add_rmsnorm: empty operand");
+                               int out_dtype, const int* rows, int n_out, int T, int ld, int groups, hipStream_t st) {
+    SPY_REQUIRE(n_out > 0 && T > 0 && ld > 0, "spy_add_rmsnorm: empty operand");
+    SPY_REQUIRE(groups > 0 && groups <= 65535 && ld % groups == 0, "spy_add_rmsnorm: %d groups do not divide rows of %d", groups, ld);
     SPY_REQUIRE(delta || !delta2, "spy_add_rmsnorm: a second addend without a first");
+    const int H = ld / groups;
+    const dim3 grid(n_out, groups);
     const int threads = H >= 2048 ? 256 : (H >= 512 ? 128 : 64);
     const bool aligned = H % 4 == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)delta % 16) == 0 && ((uintptr_t)delta2 % 16) == 0 && ((uintptr_t)w % 16) == 0 &&
                          ((uintptr_t)out % 16) == 0;
     const bool vec = aligned && H <= threads * 4 * NORM_PASSES;
     if (vec) {
-        SPY_DISPATCH(out_dtype, TA, SPY_DISPATCH(w_dtype, TW, (add_rmsnorm_kernel<TA, TW, true><<<n_out, threads, 0, st>>>(
-            resid, (const TA*)delta, (const TA*)delta2, (const TW*)w, eps, (TA*)out, rows, T, H))));
+        SPY_DISPATCH(out_dtype, TA, SPY_DISPATCH(w_dtype, TW, (add_rmsnorm_kernel<TA, TW, true><<<grid, threads, 0, st>>>(
+            resid, (const TA*)delta, (const TA*)delta2, (const TW*)w, eps, (TA*)out, rows, T, H, ld))));
     } else {
-        SPY_DISPATCH(out_dtype, TA, SPY_DISPATCH(w_dtype, TW, (add_rmsnorm_kernel<TA, TW, false><<<n_out, 512, 0, st>>>(
-            resid, (const TA*)delta, (const TA*)delta2, (const TW*)w, eps, (TA*)out, rows, T, H))));
+        SPY_DISPATCH(out_dtype, TA, SPY_DISPATCH(w_dtype, TW, (add_rmsnorm_kernel<TA, TW, false><<<grid, 512, 0, st>>>(
+            resid, (const TA*)delta, (const TA*)delta2, (const TW*)w, eps, (TA*)out, rows, T, H, ld))));
     }
     SPY_CHECK_LAUNCH("spy_add_rmsnorm");
     return 0;

@@ -35,11 +35,11 @@ __device__ __forceinline__ float quad_sum(float x) {
     return x;
 }
 
-// out[t, h, j] = o[t, h, j] / sqrt(mean_j(o[t, h, :]^2) + eps) * w[(per_head ? h dv : 0) + j] * sigmoid(gate[t, h dv + j]);
-// one block per (token, head)
+// out[t, h, j] = o[t, h, j] / sqrt(mean_j(o[t, h, :]^2) + eps) * w[(per_head ? h dv : 0) + j] * sigmoid(gate[t, h dv + j])
+// (silu != 0: times silu(gate) = gate sigmoid(gate)); one block per (token, head)
 template <typename TA, typename TW>
 __global__ void head_norm_gate_kernel(TA* __restrict__ out, const float* __restrict__ o, const TA* __restrict__ gate, long long gs,
-                                      const TW* __restrict__ w, int per_head, float eps, int H, int dv) {
+                                      const TW* __restrict__ w, int per_head, float eps, int H, int dv, int silu = 0) {
     __shared__ float red[16];
     const int t = blockIdx.x, h = blockIdx.y;
     const float* row = o + ((size_t)t * H + h) * dv;
@@ -50,8 +50,10 @@ __global__ void head_norm_gate_kernel(TA* __restrict__ out, const float* __restr
     const TA* g = gate + (size_t)t * gs + (size_t)h * dv;
     const TW* wr = w + (per_head ? (size_t)h * dv : 0);
     TA* dst = out + ((size_t)t * H + h) * dv;
-    for (int j = threadIdx.x; j < dv; j += blockDim.x)
-        dst[j] = from_f32<TA>(((row[j] * r) * to_f32<TW>(wr[j])) * mm_sigmoid(to_f32<TA>(g[j])));
+    for (int j = threadIdx.x; j < dv; j += blockDim.x) {
+        const float gj = to_f32<TA>(g[j]);
+        dst[j] = from_f32<TA>(((row[j] * r) * to_f32<TW>(wr[j])) * (silu ? gj * mm_sigmoid(gj) : mm_sigmoid(gj)));
+    }
 }
 
 // ---- mLSTM ----------------------------------------------------------------------------------------------------------
@@ -468,7 +470,8 @@ extern "C" int spy_causal_conv_silu(void* y, const void* x, long long xs, int dt
 template <typename TA, typename TW>
 __global__ __launch_bounds__(64) void delta_prepare_kernel(float* __restrict__ qk, const TA* __restrict__ qkv, float* __restrict__ beta,
                                                           float* __restrict__ dec, const TW* __restrict__ a_log,
-                                                          const TW* __restrict__ dt_bias, int H, int G, int d, int dv) {
+                                                          const TW* __restrict__ dt_bias, int H, int G, int d, int dv, int dd) {
+    // dd: decays per head, d (one per key channel) or 1 (one for the head)
     const int t = blockIdx.x, unit = blockIdx.y, lane = threadIdx.x;
     const int C = 2 * G * d + H * dv;
     if (unit < G) {
@@ -493,8 +496,8 @@ __global__ __launch_bounds__(64) void delta_prepare_kernel(float* __restrict__ q
     }
     const int h = unit - G;
     const float rate = expf(to_f32<TW>(a_log[h]));
-    float* z = dec + ((size_t)t * H + h) * d;
-    for (int i = lane; i < d; i += 64) z[i] = expf(-rate * softplus_f(z[i] + to_f32<TW>(dt_bias[(size_t)h * d + i])));
+    float* z = dec + ((size_t)t * H + h) * dd;
+    for (int i = lane; i < dd; i += 64) z[i] = expf(-rate * softplus_f(z[i] + to_f32<TW>(dt_bias[(size_t)h * dd + i])));
     if (lane == 0) beta[(size_t)t * H + h] = mm_sigmoid(beta[(size_t)t * H + h]);
 }
 
@@ -502,7 +505,7 @@ template <typename TA, typename TW, int DR>
 __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
     float* __restrict__ o_out, float* __restrict__ state, long long state_stride, const TA* __restrict__ qkv, const float* __restrict__ qk,
     const float* __restrict__ beta_pre, const float* __restrict__ dec_pre, const int* __restrict__ cu_q,
-    const int* __restrict__ slot_ids, int num_slots, int H, int G, int d, int dv) {
+    const int* __restrict__ slot_ids, int num_slots, int H, int G, int d, int dv, int dd) {
     constexpr int R = (DR + MM_SLICE - 1) / MM_SLICE, LD = R * MM_SLICE, DQ = DR / 4;
     __shared__ __align__(16) float ks[LD], qs[LD], dec[LD];
     const int s = blockIdx.x, h = blockIdx.y, c = blockIdx.z, lane = threadIdx.x;
@@ -533,7 +536,7 @@ __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
             const int idx = lane + MM_SLICE * i;                                                 \
             qr[U][i] = idx < d ? qk_[(size_t)g * d + idx] : 0.f;                                 \
             kr[U][i] = idx < d ? qk_[(size_t)(G + g) * d + idx] : 0.f;                           \
-            zr[U][i] = idx < d ? dec_pre[((size_t)(TT) * H + h) * d + idx] : 1.f;                \
+            zr[U][i] = idx < d ? dec_pre[((size_t)(TT) * H + h) * dd + (dd == 1 ? 0 : idx)] : 1.f; \
         }                                                                                        \
         vr[U] = col ? to_f32<TA>(qkv[(size_t)(TT) * C + (size_t)2 * G * d + (size_t)h * dv + j]) : 0.f; \
         br[U] = beta_pre[(size_t)(TT) * H + h];                                                  \
@@ -587,23 +590,237 @@ __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
 extern "C" int spy_delta_rule(void* out, float* o_tmp, float* qk_tmp, float* state, long long state_stride, const void* qkv, int dtype,
                               float* beta_pre, float* dec_pre, const void* a_log, const void* dt_bias, int w_dtype, const void* gate, long long gs,
                               const void* norm_w, float eps, const int* cu_q, const int* slot_ids, int num_slots, int S, int T, int H,
-                              int G, int d, int dv, hipStream_t st) {
+                              int G, int d, int dv, int dd, int silu_gate, hipStream_t st) {
     SPY_REQUIRE(S > 0 && T > 0 && H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0 && num_slots > 0 && o_tmp, "spy_delta_rule: empty operand");
+    SPY_REQUIRE(dd == d || dd == 1, "spy_delta_rule: %d decays for a head of %d key channels (one, or one per channel)", dd, d);
     SPY_REQUIRE(d <= 256 && dv <= 1024 && H <= 65535, "spy_delta_rule: heads of %d x %d (key size up to 256, value size up to 1024)", d, dv);
     SPY_REQUIRE(state_stride >= (long long)H * d * dv && gs >= (long long)H * dv, "spy_delta_rule: the state or the gate rows are too short");
     SPY_REQUIRE(qk_tmp && G + H <= 65535, "spy_delta_rule: no room for the unit vectors");
     const dim3 pgrid(T, G + H);
     SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (delta_prepare_kernel<TA, TW><<<pgrid, 64, 0, st>>>(
-        qk_tmp, (const TA*)qkv, beta_pre, dec_pre, (const TW*)a_log, (const TW*)dt_bias, H, G, d, dv))));
+        qk_tmp, (const TA*)qkv, beta_pre, dec_pre, (const TW*)a_log, (const TW*)dt_bias, H, G, d, dv, dd))));
     SPY_CHECK_LAUNCH("spy_delta_rule (unit vectors and decays)");
     const dim3 grid(S, H, (dv + MM_COLS - 1) / MM_COLS);
     SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, MM_LAUNCH(delta_rule_kernel, o_tmp, state, state_stride, (const TA*)qkv, qk_tmp, beta_pre,
-        dec_pre, cu_q, slot_ids, num_slots, H, G, d, dv)));
+        dec_pre, cu_q, slot_ids, num_slots, H, G, d, dv, dd)));
     SPY_CHECK_LAUNCH("spy_delta_rule");
     const dim3 ngrid(T, H);
     const int nthreads = dv >= 256 ? 256 : 64;
     SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (head_norm_gate_kernel<TA, TW><<<ngrid, nthreads, 0, st>>>(
-        (TA*)out, o_tmp, (const TA*)gate, gs, (const TW*)norm_w, 0, eps, H, dv))));
+        (TA*)out, o_tmp, (const TA*)gate, gs, (const TW*)norm_w, 0, eps, H, dv, silu_gate))));
     SPY_CHECK_LAUNCH("spy_delta_rule (norm and gate)");
+    return 0;
+}
+
+// ---- token shift -------------------------------------------------------------------------------------------------------
+// out[s][t][c] = x[t][c] + (x'[t][c] - x[t][c]) mu[s][c], x' the row before t in its request: the entry's row before, or,
+// for an entry's first token, the request's kept row (float32, `keep_stride` values from slot to slot).  A second kernel
+// then leaves every entry's last row as the request's kept row (after all reads of the old one: the next launch).
+template <typename TA, typename TW>
+__global__ void token_shift_kernel(TA* __restrict__ out, const TA* __restrict__ x, const TW* __restrict__ mu, int n,
+                                   const float* __restrict__ keep, long long keep_stride, const int* __restrict__ token_entry,
+                                   const int* __restrict__ cu_q, const int* __restrict__ slot_ids, int num_slots, int T, int W) {
+    const size_t total = (size_t)T * W;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const int t = (int)(i / W), c = (int)(i - (size_t)t * W);
+        const int e = token_entry[t];
+        float prev;
+        if (t > cu_q[e]) prev = to_f32<TA>(x[i - W]);
+        else {
+            const int slot = slot_ids[e];
+            prev = (slot >= 0 && slot < num_slots) ? keep[(size_t)slot * keep_stride + c] : 0.f;
+        }
+        const float cur = to_f32<TA>(x[i]);
+        for (int s = 0; s < n; ++s) out[(size_t)s * total + i] = from_f32<TA>(fmaf(prev - cur, to_f32<TW>(mu[(size_t)s * W + c]), cur));
+    }
+}
+
+template <typename TA>
+__global__ void shift_keep_kernel(float* __restrict__ keep, long long keep_stride, const TA* __restrict__ x, const int* __restrict__ cu_q,
+                                  const int* __restrict__ slot_ids, int num_slots, int W) {
+    const int s = blockIdx.y;
+    const int slot = slot_ids[s];
+    const int last = cu_q[s + 1] - 1;
+    if (slot < 0 || slot >= num_slots || last < cu_q[s]) return;
+    for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < W; c += gridDim.x * blockDim.x)
+        keep[(size_t)slot * keep_stride + c] = to_f32<TA>(x[(size_t)last * W + c]);
+}
+
+extern "C" int spy_token_shift(void* out, const void* x, int dtype, const void* mu, int w_dtype, int n, float* keep, long long keep_stride,
+                               const int* token_entry, const int* cu_q, const int* slot_ids, int num_slots, int S, int T, int W,
+                               hipStream_t st) {
+    SPY_REQUIRE(S > 0 && T > 0 && W > 0 && n > 0 && num_slots > 0 && keep && keep_stride >= W && S <= 65535, "spy_token_shift: bad sizes");
+    const size_t total = (size_t)T * W;
+    const unsigned blocks = (unsigned)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256);
+    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (token_shift_kernel<TA, TW><<<blocks, 256, 0, st>>>(
+        (TA*)out, (const TA*)x, (const TW*)mu, n, keep, keep_stride, token_entry, cu_q, slot_ids, num_slots, T, W))));
+    SPY_CHECK_LAUNCH("spy_token_shift");
+    const dim3 kgrid((W + 255) / 256, S);
+    SPY_DISPATCH(dtype, TA, (shift_keep_kernel<TA><<<kgrid, 256, 0, st>>>(keep, keep_stride, (const TA*)x, cu_q, slot_ids, num_slots, W)));
+    SPY_CHECK_LAUNCH("spy_token_shift (kept row)");
+    return 0;
+}
+
+__global__ void tanh_kernel(float* __restrict__ x, long long n) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) x[i] = tanhf(x[i]);
+}
+
+extern "C" int spy_tanh(float* x, long long n, hipStream_t st) {
+    SPY_REQUIRE(n > 0, "spy_tanh: empty operand");
+    const unsigned blocks = (unsigned)((n + 255) / 256 > 65536 ? 65536 : (n + 255) / 256);
+    tanh_kernel<<<blocks, 256, 0, st>>>(x, n);
+    SPY_CHECK_LAUNCH("spy_tanh");
+    return 0;
+}
+
+// ---- a state with a decay per key channel, read before the write, and a bonus for the token's own pair ------------------
+// r, k, v, gate [T, H d]; dec [T, H d] float32: raw products, turned in place into the decays w = exp(-exp(. + w0));
+// bonus [T, H] = sum_i r_i u_i k_i.  Per head: o_j = sum_i r_i S_ij + bonus v_j; S_ij = w_i S_ij + k_i v_j.
+// state [slots][stride]: S of head h at h d d, row (key channel) i and column j at i d + j.
+// The preparation, for all tokens at once: one wave per (token, head).
+template <typename TA, typename TW>
+__global__ __launch_bounds__(64) void time_mix_prepare_kernel(float* __restrict__ dec, float* __restrict__ bonus, const TA* __restrict__ r,
+                                                             const TA* __restrict__ k, const TW* __restrict__ w0, const TW* __restrict__ u,
+                                                             int H, int d) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const size_t at = ((size_t)t * H + h) * d;
+    float b = 0.f;
+    for (int i = lane; i < d; i += 64) {
+        dec[at + i] = expf(-expf(dec[at + i] + to_f32<TW>(w0[(size_t)h * d + i])));
+        b = fmaf(to_f32<TA>(r[at + i]) * to_f32<TW>(u[(size_t)h * d + i]), to_f32<TA>(k[at + i]), b);
+    }
+    b = wave_sum(b);
+    if (lane == 0) bonus[(size_t)t * H + h] = b;
+}
+
+// The walk: one wave per (entry, head, slice of 16 value channels), four lanes a column, as the delta rule's.
+template <typename TA, typename TW, int DR>
+__global__ __launch_bounds__(MM_SLICE) void time_mix_kernel(
+    float* __restrict__ o_out, float* __restrict__ state, long long state_stride, const TA* __restrict__ r, const TA* __restrict__ k,
+    const TA* __restrict__ v, const float* __restrict__ dec_in, const float* __restrict__ bonus, const int* __restrict__ cu_q,
+    const int* __restrict__ slot_ids, int num_slots, int H, int d) {
+    constexpr int R = (DR + MM_SLICE - 1) / MM_SLICE, LD = R * MM_SLICE, DQ = DR / 4;
+    __shared__ __align__(16) float ks[LD], rs[LD], dec[LD];
+    const int s = blockIdx.x, h = blockIdx.y, c = blockIdx.z, lane = threadIdx.x;
+    const int part = lane & 3, j = c * MM_COLS + (lane >> 2);
+    const int row0 = part * DQ;
+    const int slot = slot_ids[s];
+    if (slot < 0 || slot >= num_slots) return;
+    float* st = state + (size_t)slot * state_stride + (size_t)h * d * d;
+    const bool col = j < d;
+    // (rows beyond d: S zero, staged k and r zero, decay one; the loops run over all of a lane's rows without conditions)
+    float S[DQ];
+#pragma unroll
+    for (int i = 0; i < DQ; ++i) S[i] = (col && row0 + i < d) ? st[(size_t)(row0 + i) * d + j] : 0.f;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        ks[lane + MM_SLICE * i] = 0.f;
+        rs[lane + MM_SLICE * i] = 0.f;
+        dec[lane + MM_SLICE * i] = 1.f;
+    }
+    const int N = H * d;
+    const int t0 = cu_q[s], t1 = cu_q[s + 1];
+    float kr[MM_AHEAD][R], rr[MM_AHEAD][R], zr[MM_AHEAD][R], vr[MM_AHEAD], br[MM_AHEAD];
+#define TMIX_LOAD(U, TT)                                                                         \
+    if ((TT) < t1) {                                                                             \
+        const size_t at_ = (size_t)(TT) * N + (size_t)h * d;                                     \
+        _Pragma("unroll") for (int i = 0; i < R; ++i) {                                          \
+            const int idx = lane + MM_SLICE * i;                                                 \
+            rr[U][i] = idx < d ? to_f32<TA>(r[at_ + idx]) : 0.f;                                 \
+            kr[U][i] = idx < d ? to_f32<TA>(k[at_ + idx]) : 0.f;                                 \
+            zr[U][i] = idx < d ? dec_in[at_ + idx] : 1.f;                                        \
+        }                                                                                        \
+        vr[U] = col ? to_f32<TA>(v[at_ + j]) : 0.f;                                              \
+        br[U] = bonus[(size_t)(TT) * H + h];                                                     \
+    }
+#pragma unroll
+    for (int u = 0; u < MM_AHEAD; ++u) TMIX_LOAD(u, t0 + u)
+    for (int tb = t0; tb < t1; tb += MM_AHEAD) {
+#pragma unroll
+        for (int u = 0; u < MM_AHEAD; ++u) {
+            const int t = tb + u;
+            if (t < t1) {
+#pragma unroll
+                for (int i = 0; i < R; ++i) {
+                    const int idx = lane + MM_SLICE * i;
+                    if (idx < d) { rs[idx] = rr[u][i]; ks[idx] = kr[u][i]; dec[idx] = zr[u][i]; }
+                }
+                const float vj = vr[u];
+                mm_wave_order();
+                float acc = 0.f, acc2 = 0.f;
+#pragma unroll
+                for (int i = 0; i < DQ; i += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4*>(ks + row0 + i), g4 = *reinterpret_cast<const float4*>(dec + row0 + i);
+                    const float4 r4 = *reinterpret_cast<const float4*>(rs + row0 + i);
+                    acc = fmaf(S[i], r4.x, acc);          S[i] = fmaf(S[i], g4.x, k4.x * vj);
+                    acc2 = fmaf(S[i + 1], r4.y, acc2);    S[i + 1] = fmaf(S[i + 1], g4.y, k4.y * vj);
+                    acc = fmaf(S[i + 2], r4.z, acc);      S[i + 2] = fmaf(S[i + 2], g4.z, k4.z * vj);
+                    acc2 = fmaf(S[i + 3], r4.w, acc2);    S[i + 3] = fmaf(S[i + 3], g4.w, k4.w * vj);
+                }
+                acc = quad_sum(acc + acc2);
+                if (col && part == 0) o_out[(size_t)t * N + (size_t)h * d + j] = fmaf(br[u], vj, acc);
+                mm_wave_order();
+                TMIX_LOAD(u, t + MM_AHEAD)
+            }
+        }
+    }
+#undef TMIX_LOAD
+#pragma unroll
+    for (int i = 0; i < DQ; ++i)
+        if (col && row0 + i < d) st[(size_t)(row0 + i) * d + j] = S[i];
+}
+
+extern "C" int spy_time_mix(void* out, float* o_tmp, float* bonus, float* state, long long state_stride, const void* r, const void* k,
+                            const void* v, const void* gate, int dtype, float* dec_pre, const void* w0, const void* u, const void* norm_w,
+                            int w_dtype, float eps, const int* cu_q, const int* slot_ids, int num_slots, int S, int T, int H, int d,
+                            hipStream_t st) {
+    SPY_REQUIRE(S > 0 && T > 0 && H > 0 && d > 0 && num_slots > 0 && o_tmp && bonus, "spy_time_mix: empty operand");
+    SPY_REQUIRE(d <= 256 && H <= 65535, "spy_time_mix: heads of %d (up to 256)", d);
+    SPY_REQUIRE(state_stride >= (long long)H * d * d, "spy_time_mix: the state is too short");
+    const dim3 pgrid(T, H);
+    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (time_mix_prepare_kernel<TA, TW><<<pgrid, 64, 0, st>>>(
+        dec_pre, bonus, (const TA*)r, (const TA*)k, (const TW*)w0, (const TW*)u, H, d))));
+    SPY_CHECK_LAUNCH("spy_time_mix (decays and bonus)");
+    const dim3 grid(S, H, (d + MM_COLS - 1) / MM_COLS);
+    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, MM_LAUNCH(time_mix_kernel, o_tmp, state, state_stride, (const TA*)r, (const TA*)k,
+        (const TA*)v, dec_pre, bonus, cu_q, slot_ids, num_slots, H, d)));
+    SPY_CHECK_LAUNCH("spy_time_mix");
+    const dim3 ngrid(T, H);
+    const int nthreads = d >= 256 ? 256 : 64;
+    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (head_norm_gate_kernel<TA, TW><<<ngrid, nthreads, 0, st>>>(
+        (TA*)out, o_tmp, (const TA*)gate, (long long)H * d, (const TW*)norm_w, 1, eps, H, d, 1))));
+    SPY_CHECK_LAUNCH("spy_time_mix (norm and gate)");
+    return 0;
+}
+
+// ---- two results normed over the width and averaged ----------------------------------------------------------------------
+// out[t] = (a[t] / rms(a[t]) * wa + b[t] / rms(b[t]) * wb) / 2; one block per row
+template <typename TA, typename TW>
+__global__ void norm_pair_mean_kernel(TA* __restrict__ out, const TA* __restrict__ a, const TA* __restrict__ b, const TW* __restrict__ wa,
+                                      const TW* __restrict__ wb, float eps, int W) {
+    __shared__ float red[16];
+    const TA* ar = a + (size_t)blockIdx.x * W;
+    const TA* br = b + (size_t)blockIdx.x * W;
+    float sa = 0.f, sb = 0.f;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+        const float x = to_f32<TA>(ar[i]), y = to_f32<TA>(br[i]);
+        sa = fmaf(x, x, sa);
+        sb = fmaf(y, y, sb);
+    }
+    sa = block_sum(sa, red);
+    sb = block_sum(sb, red);
+    const float ra = 0.5f / sqrtf(sa / (float)W + eps), rb = 0.5f / sqrtf(sb / (float)W + eps);
+    TA* o = out + (size_t)blockIdx.x * W;
+    for (int i = threadIdx.x; i < W; i += blockDim.x)
+        o[i] = from_f32<TA>(fmaf(to_f32<TA>(ar[i]) * ra, to_f32<TW>(wa[i]), (to_f32<TA>(br[i]) * rb) * to_f32<TW>(wb[i])));
+}
+
+extern "C" int spy_norm_pair_mean(void* out, const void* a, const void* b, int dtype, const void* wa, const void* wb, int w_dtype, float eps,
+                                  int T, int W, hipStream_t st) {
+    SPY_REQUIRE(T > 0 && W > 0, "spy_norm_pair_mean: empty operand");
+    const int threads = W >= 1024 ? 256 : 64;
+    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (norm_pair_mean_kernel<TA, TW><<<T, threads, 0, st>>>(
+        (TA*)out, (const TA*)a, (const TA*)b, (const TW*)wa, (const TW*)wb, eps, W))));
+    SPY_CHECK_LAUNCH("spy_norm_pair_mean");
     return 0;
 }

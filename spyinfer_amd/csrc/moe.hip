@@ -8,7 +8,8 @@
 //            correction) over their sum (+ 1e-20), times `scale`.
 //   align:   rows of the sorted order: expert e's pairs in a run that starts at a multiple of MOE_TM rows, padded with -1.
 //   gemm:    C[row] = A[source of row] . W[expert of the row's tile]^T, float32 products and sums; optionally gated:
-//            W = [gate rows | up rows], C = silu(gate) * up.
+//            W = [gate rows | up rows], C = silu(gate) * up; or (MoeAct kind 1) with the row's weight w multiplied into both
+//            sums first, g = min(w gate, limit), u = clamp(w up, -limit, limit), C = g sigmoid(1.702 g) (u + 1).
 //   combine: out[t] = sum_k weight[t, k] * Y[row of pair (t, k)].
 #include "common.h"
 #include <math.h>
@@ -16,27 +17,48 @@
 #define MOE_TM 16
 #define MOE_MAX_EXPERTS 1024
 
+// What a gated product does with its two sums (see the top).  pair_w: the weight of every (token, choice) pair, or null.
+struct MoeAct {
+    int kind;
+    float limit;
+    const float* pair_w;
+};
+__device__ __forceinline__ float moe_gated(float g, float u, const MoeAct& a, float w) {
+    if (a.kind == 0) return g / (1.0f + expf(-g)) * u;
+    g = fminf(g * w, a.limit);
+    u = fminf(fmaxf(u * w, -a.limit), a.limit);
+    return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+}
+
 // one wave per token
 __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ ids, float* __restrict__ weights, const float* __restrict__ z,
                                                        const float* __restrict__ correction, int E, int top, int groups, int keep,
-                                                       float scale) {
+                                                       float scale, int sigmoid, int renorm) {
     __shared__ float sc[MOE_MAX_EXPERTS], ch[MOE_MAX_EXPERTS], gsc[MOE_MAX_EXPERTS];
     __shared__ int allowed[MOE_MAX_EXPERTS], sel[MOE_MAX_EXPERTS];
     const int t = blockIdx.x, lane = threadIdx.x;
     const float* zr = z + (size_t)t * E;
-    float mx = -INFINITY;
-    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, zr[e]);
-    mx = wave_max(mx);
-    float sum = 0.f;
-    for (int e = lane; e < E; e += 64) {
-        const float p = expf(zr[e] - mx);
-        sc[e] = p;
-        sum += p;
-    }
-    sum = wave_sum(sum);
-    for (int e = lane; e < E; e += 64) {
-        sc[e] = sc[e] / sum;
-        ch[e] = sc[e] + correction[e];
+    if (sigmoid) {
+        // every logit by itself
+        for (int e = lane; e < E; e += 64) {
+            sc[e] = 1.0f / (1.0f + expf(-zr[e]));
+            ch[e] = sc[e] + (correction ? correction[e] : 0.f);
+        }
+    } else {
+        float mx = -INFINITY;
+        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, zr[e]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int e = lane; e < E; e += 64) {
+            const float p = expf(zr[e] - mx);
+            sc[e] = p;
+            sum += p;
+        }
+        sum = wave_sum(sum);
+        for (int e = lane; e < E; e += 64) {
+            sc[e] = sc[e] / sum;
+            ch[e] = sc[e] + (correction ? correction[e] : 0.f);
+        }
     }
     __syncthreads();
     const int per = E / groups;
@@ -82,7 +104,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ ids, fl
         if (lane == 0) { ch[bi] = -INFINITY; sel[r] = bi; }
         __syncthreads();
     }
-    const float norm = scale / (wsum + 1e-20f);
+    const float norm = renorm ? scale / (wsum + 1e-20f) : scale;
     for (int r = lane; r < top; r += 64) {
         ids[(size_t)t * top + r] = sel[r];
         weights[(size_t)t * top + r] = sc[sel[r]] * norm;
@@ -90,11 +112,11 @@ __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ ids, fl
 }
 
 extern "C" int spy_moe_route(int* ids, float* weights, const float* z, const float* correction, int T, int E, int top, int groups,
-                             int keep, float scale, hipStream_t st) {
+                             int keep, float scale, int sigmoid, int renorm, hipStream_t st) {
     SPY_REQUIRE(T > 0 && E > 0 && E <= MOE_MAX_EXPERTS, "spy_moe_route: %d experts (1..%d)", E, MOE_MAX_EXPERTS);
     SPY_REQUIRE(groups > 0 && E % groups == 0 && keep > 0 && keep <= groups && top > 0 && top <= keep * (E / groups),
                 "spy_moe_route: %d of %d groups of %d experts cannot give %d choices", keep, groups, E / (groups > 0 ? groups : 1), top);
-    moe_route_kernel<<<T, 64, 0, st>>>(ids, weights, z, correction, E, top, groups, keep, scale);
+    moe_route_kernel<<<T, 64, 0, st>>>(ids, weights, z, correction, E, top, groups, keep, scale, sigmoid, renorm);
     SPY_CHECK_LAUNCH("spy_moe_route");
     return 0;
 }
@@ -157,7 +179,7 @@ extern "C" int spy_moe_tile_rows() { return MOE_TM; }
 template <typename TA, typename TW, typename TC, bool GATED>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(TC* __restrict__ C, const TA* __restrict__ A, const TW* __restrict__ W,
                                                        const int* __restrict__ tile_expert, const int* __restrict__ sorted_pair,
-                                                       int gather, int N, int K, long long w_stride) {
+                                                       int gather, int N, int K, long long w_stride, MoeAct act) {
     __shared__ float As[MG_K][MOE_TM + 1];
     __shared__ float Ws[GATED ? 2 : 1][MG_K][MG_TN + 4];
     __shared__ int src[MOE_TM];
@@ -201,13 +223,14 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(TC* __restrict__ C, const
     }
     if (src[ty] < 0) return;
     const size_t row = (size_t)tile * MOE_TM + ty;
+    const float rw = (GATED && act.pair_w) ? act.pair_w[sorted_pair[row]] : 1.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int n = n0 + tx * 4 + i;
         if (n >= N) continue;
         float v = acc[i];
         if (GATED) {
-            v = acc[i] / (1.0f + expf(-acc[i])) * acc2[i];
+            v = moe_gated(acc[i], acc2[i], act, rw);
         }
         C[row * N + n] = from_f32<TC>(v);
     }
@@ -227,7 +250,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float moe_f32x4_t;
 template <int MT, bool GATED, typename TC>
 __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(TC* __restrict__ C, const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
                                                             const int* __restrict__ tile_expert, const int* __restrict__ sorted_pair,
-                                                            int gather, int max_tiles, int N, int K, long long w_stride) {
+                                                            int gather, int max_tiles, int N, int K, long long w_stride, MoeAct act) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int r = lane & 15, g = lane >> 4;
     constexpr int NT = 2;
@@ -305,13 +328,11 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(TC* __restrict__ C, 
             if (mt >= run || !xok[mt]) continue;
             const size_t row = (size_t)(t + mt) * MOE_TM + r;
             if (GATED) {
+                const float rw = act.pair_w ? act.pair_w[sorted_pair[row]] : 1.f;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int col = n0 + 4 * g + i;
-                    if (col < N) {
-                        const float gt = acc[0][mt][i];
-                        C[row * N + col] = from_f32<TC>(gt / (1.0f + expf(-gt)) * acc[1][mt][i]);
-                    }
+                    if (col < N) C[row * N + col] = from_f32<TC>(moe_gated(acc[0][mt][i], acc[1][mt][i], act, rw));
                 }
             } else {
 #pragma unroll
@@ -336,7 +357,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(TC* __restrict__ C, 
 template <bool GATED, typename TC>
 __global__ __launch_bounds__(256) void moe_gemm_mfma_lds_kernel(TC* __restrict__ C, const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
                                                                 const int* __restrict__ tile_expert, const int* __restrict__ sorted_pair,
-                                                                int gather, int max_tiles, int N, int K, long long w_stride) {
+                                                                int gather, int max_tiles, int N, int K, long long w_stride, MoeAct act) {
     constexpr int MT = 8, NT = 2;
     __shared__ __align__(16) bf16_t xs[MOE_ROWS * MOE_LDS_STRIDE];
     __shared__ int src_row[MOE_ROWS];
@@ -426,13 +447,11 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_lds_kernel(TC* __restrict__
                 if (mt >= run || !xok[mt]) continue;
                 const size_t row = (size_t)(t + mt) * MOE_TM + r;
                 if (GATED) {
+                    const float rw = act.pair_w ? act.pair_w[sorted_pair[row]] : 1.f;
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int col = n0 + 4 * g + i;
-                        if (col < N) {
-                            const float gt = acc[0][mt][i];
-                            C[row * N + col] = from_f32<TC>(gt / (1.0f + expf(-gt)) * acc[1][mt][i]);
-                        }
+                        if (col < N) C[row * N + col] = from_f32<TC>(moe_gated(acc[0][mt][i], acc[1][mt][i], act, rw));
                     }
                 } else {
 #pragma unroll
@@ -451,7 +470,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_lds_kernel(TC* __restrict__
 
 template <int MT>
 static int moe_gemm_mfma_launch(void* C, int c_dtype, const void* A, const void* W, const int* tile_expert, const int* sorted_pair,
-                                int gather, int gated, int max_tiles, int N, int K, hipStream_t st) {
+                                int gather, int gated, int max_tiles, int N, int K, MoeAct act, hipStream_t st) {
     const long long ws = (long long)(gated ? 2 : 1) * N * K;
     const int cols = gated ? 64 : 128;
     const dim3 grid((max_tiles + MT - 1) / MT, (N + cols - 1) / cols);
@@ -459,29 +478,31 @@ static int moe_gemm_mfma_launch(void* C, int c_dtype, const void* A, const void*
     if (MT == 8) {
         if (gated) {
             SPY_DISPATCH(c_dtype, TC, (moe_gemm_mfma_lds_kernel<true, TC><<<grid, 256, 0, st>>>((TC*)C, (const bf16_t*)A, (const bf16_t*)W, tile_expert,
-                                                                                               sorted_pair, gather, max_tiles, N, K, ws)));
+                                                                                               sorted_pair, gather, max_tiles, N, K, ws, act)));
         } else {
             SPY_DISPATCH(c_dtype, TC, (moe_gemm_mfma_lds_kernel<false, TC><<<grid, 256, 0, st>>>((TC*)C, (const bf16_t*)A, (const bf16_t*)W, tile_expert,
-                                                                                                sorted_pair, gather, max_tiles, N, K, ws)));
+                                                                                                sorted_pair, gather, max_tiles, N, K, ws, act)));
         }
     } else if (gated) {
         SPY_DISPATCH(c_dtype, TC, (moe_gemm_mfma_kernel<MT, true, TC><<<grid, 256, 0, st>>>((TC*)C, (const bf16_t*)A, (const bf16_t*)W, tile_expert,
-                                                                                           sorted_pair, gather, max_tiles, N, K, ws)));
+                                                                                           sorted_pair, gather, max_tiles, N, K, ws, act)));
     } else {
         SPY_DISPATCH(c_dtype, TC, (moe_gemm_mfma_kernel<MT, false, TC><<<grid, 256, 0, st>>>((TC*)C, (const bf16_t*)A, (const bf16_t*)W, tile_expert,
-                                                                                            sorted_pair, gather, max_tiles, N, K, ws)));
+                                                                                            sorted_pair, gather, max_tiles, N, K, ws, act)));
     }
     return 0;
 }
 
 extern "C" int spy_moe_gemm(void* C, int c_dtype, const void* A, int a_dtype, const void* W, int w_dtype, const int* tile_expert,
                             const int* sorted_pair, int gather, int gated, int max_tiles, int E, int N, int K, int tiles_per_block,
-                            hipStream_t st) {
+                            int act_kind, float limit, const float* pair_w, hipStream_t st) {
     SPY_REQUIRE(max_tiles > 0 && E > 0 && N > 0 && K > 0 && gather >= 0, "spy_moe_gemm: bad sizes (%d tiles)", max_tiles);
+    SPY_REQUIRE((act_kind == 0 && !pair_w) || (act_kind == 1 && gated && limit > 0.f), "spy_moe_gemm: activation %d with limit %g", act_kind, (double)limit);
+    const MoeAct act = {act_kind, limit, pair_w};
     // bfloat16 operands in 16-byte pieces: the matrix cores; tiles_per_block: 0 = the plain float32 kernel
     if (tiles_per_block > 0 && a_dtype == SPY_BF16 && w_dtype == SPY_BF16 && K % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0) {
-        const int rc = tiles_per_block >= 8 ? moe_gemm_mfma_launch<8>(C, c_dtype, A, W, tile_expert, sorted_pair, gather, gated, max_tiles, N, K, st)
-                                            : moe_gemm_mfma_launch<1>(C, c_dtype, A, W, tile_expert, sorted_pair, gather, gated, max_tiles, N, K, st);
+        const int rc = tiles_per_block >= 8 ? moe_gemm_mfma_launch<8>(C, c_dtype, A, W, tile_expert, sorted_pair, gather, gated, max_tiles, N, K, act, st)
+                                            : moe_gemm_mfma_launch<1>(C, c_dtype, A, W, tile_expert, sorted_pair, gather, gated, max_tiles, N, K, act, st);
         if (rc) return rc;
         SPY_CHECK_LAUNCH("spy_moe_gemm (mfma)");
         return 0;
@@ -491,16 +512,16 @@ extern "C" int spy_moe_gemm(void* C, int c_dtype, const void* A, int a_dtype, co
     const long long ws = (long long)(gated ? 2 : 1) * N * K;
     if (gated) {
         SPY_DISPATCH(a_dtype, TA, SPY_DISPATCH(w_dtype, TW, SPY_DISPATCH(c_dtype, TC, (moe_gemm_kernel<TA, TW, TC, true><<<grid, 256, 0, st>>>(
-            (TC*)C, (const TA*)A, (const TW*)W, tile_expert, sorted_pair, gather, N, K, ws)))));
+            (TC*)C, (const TA*)A, (const TW*)W, tile_expert, sorted_pair, gather, N, K, ws, act)))));
     } else {
         SPY_DISPATCH(a_dtype, TA, SPY_DISPATCH(w_dtype, TW, SPY_DISPATCH(c_dtype, TC, (moe_gemm_kernel<TA, TW, TC, false><<<grid, 256, 0, st>>>(
-            (TC*)C, (const TA*)A, (const TW*)W, tile_expert, sorted_pair, gather, N, K, ws)))));
+            (TC*)C, (const TA*)A, (const TW*)W, tile_expert, sorted_pair, gather, N, K, ws, act)))));
     }
     SPY_CHECK_LAUNCH("spy_moe_gemm");
     return 0;
 }
 
-// out[t, :] = sum_k weights[t, k] * Y[pair_row[t top + k], :], added in ascending k
+// out[t, :] = sum_k weights[t, k] * Y[pair_row[t top + k], :], added in ascending k (no weights: all one)
 template <typename TC>
 __global__ void moe_combine_kernel(TC* __restrict__ out, const float* __restrict__ Y, const float* __restrict__ weights,
                                    const int* __restrict__ pair_row, int top, int H) {
@@ -509,7 +530,7 @@ __global__ void moe_combine_kernel(TC* __restrict__ out, const float* __restrict
         float acc = 0.f;
         for (int k = 0; k < top; ++k) {
             const int row = pair_row[(size_t)t * top + k];
-            if (row >= 0) acc = fmaf(weights[(size_t)t * top + k], Y[(size_t)row * H + c], acc);
+            if (row >= 0) acc = fmaf(weights ? weights[(size_t)t * top + k] : 1.f, Y[(size_t)row * H + c], acc);
         }
         out[(size_t)t * H + c] = from_f32<TC>(acc);
     }

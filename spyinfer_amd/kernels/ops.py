@@ -78,7 +78,8 @@ class _Hip:
                      "spy_pair_embedding", "spy_norm_residual", "spy_depth_mix", "spy_xielu", "spy_mingru", "spy_latent_prepare",
                      "spy_gemm_strided", "spy_latent_attention", "spy_latent_attention_mfma", "spy_latent_attention_mfma_workspace", "spy_head_products",
                      "spy_bias_rope_store", "spy_sigmoid_gate", "spy_mlstm", "spy_causal_conv_silu", "spy_delta_rule", "spy_moe_route",
-                     "spy_moe_align", "spy_moe_gemm", "spy_moe_combine", "spy_moe_tile_rows"):
+                     "spy_moe_align", "spy_moe_gemm", "spy_moe_combine", "spy_moe_tile_rows", "spy_token_shift", "spy_tanh", "spy_time_mix",
+                     "spy_norm_pair_mean"):
             if not hasattr(self.lib, name):
                 raise KernelError("the kernel library %s lacks %s: it is older than its sources; build it again "
                                   "(spyinfer_amd.kernels.build.build())" % (self.lib._name, name))
@@ -136,9 +137,10 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> tor
 
 
 def add_rms_norm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
-                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None, delta2: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None, delta2: Optional[torch.Tensor] = None, groups: int = 1) -> torch.Tensor:
     """resid += delta (float32, in place; skipped if delta is None), then RMS-normalise.  ``delta2``: a second addend
-    (two sublayers that read one norm): resid += delta + delta2, the two summed in float32 first.
+    (two sublayers that read one norm): resid += delta + delta2, the two summed in float32 first.  ``groups``: the row is
+    cut into that many equal consecutive parts, each over its own root mean square.
 
     Without ``rows``: every row is updated and normalised -> [T, H].  With ``rows``
     (int32 [R]): only those rows are summed and normalised -> [R, H]; resid is left as it is."""
@@ -148,6 +150,7 @@ def add_rms_norm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: tor
         _check(delta is not None and delta2.shape == delta.shape and delta2.dtype == delta.dtype, "add_rms_norm: the second addend must be like the first")
     T, H = resid.shape
     _check(weight.shape == (H,), "add_rms_norm: weight must be [H]")
+    _check(groups >= 1 and H % groups == 0, "add_rms_norm: %d groups do not divide rows of %d", groups, H)
     if delta is not None:
         _check(delta.shape == (T, H) and delta.dtype == out_dtype, "add_rms_norm: delta must be [T, H] of the activation dtype")
     if rows is not None:
@@ -157,7 +160,7 @@ def add_rms_norm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: tor
     if n_out:
         hip().call("spy_add_rmsnorm", _ptr(resid), _ptr(delta), _ptr(delta2), _ptr(weight), _code(weight, "norm weight"),
                    ctypes.c_float(eps), _ptr(out), _code(out, "norm output"), _ptr(rows), ctypes.c_int(n_out),
-                   ctypes.c_int(T), ctypes.c_int(H), _Hip.stream())
+                   ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(groups), _Hip.stream())
     return out
 
 
@@ -731,10 +734,11 @@ def fused_attention_ok(dtype, meta: AttentionMeta, n_q: int, n_kv: int, d: int, 
 
 def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: torch.Tensor, page_size: int, meta: AttentionMeta,
                     n_q: int, n_kv: int, d: int, scale: float, window: Optional[int], raw: Optional[RawQKV] = None,
-                    for_product: bool = False):
+                    for_product: bool = False, softcap: float = 0.0):
     """Causal grouped-query attention of the step's query tokens over the paged cache
     (which already holds this step's keys and values, or gets them from ``raw`` in this call).  Query at position p
-    reads keys max(0, p - window + 1) .. p.  Scores, softmax and the weighted sum are float32.
+    reads keys max(0, p - window + 1) .. p.  Scores, softmax and the weighted sum are float32.  ``softcap`` > 0: a
+    score is softcap tanh(q . k scale / softcap).
     ``for_product``: the result goes into a decode product only and may come as OperandRows (it does for steps of at
     most 128 tokens, ``attention_hands_over_operand_rows``)."""
     T, S = meta.T, meta.S
@@ -766,6 +770,8 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
     _check(meta.max_kv_len <= meta.max_blocks * page_size, "paged_attention: block tables are shorter than the longest request")
     win = 0 if window is None else int(window)
     _check(win >= 0, "paged_attention: window must be positive")
+    softcap = float(softcap or 0.0)
+    _check(softcap >= 0.0 and (raw is None or softcap == 0.0), "paged_attention: the scores' cap must not be negative (and the raw product takes none)")
     out = q if raw is not None else torch.empty_like(q)
     if T == 0:
         return out
@@ -784,7 +790,7 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
         common = (ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(meta.cu_q), _ptr(meta.pos0), _ptr(meta.kv_len),
                   _ptr(meta.block_table), ctypes.c_int(meta.max_blocks))
         sizes = (ctypes.c_int(S), ctypes.c_int(T), ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(d), ctypes.c_float(scale),
-                 ctypes.c_int(win))
+                 ctypes.c_int(win), ctypes.c_float(softcap))
         if n_big and not prefill_attention_ok(d, page_size):
             raise KernelError("paged_attention: 128-row tiles were built for head_dim %d and pages of %d, which the prefill "
                               "kernel refuses; build 16-row tiles only (ops.prefill_attention_ok)" % (d, page_size))
@@ -838,7 +844,8 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
     hip().call("spy_attention_generic", _ptr(out), _ptr(q), _code(q, "q"), _ptr(k_cache), _ptr(v_cache),
                ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(meta.kv_len), _ptr(meta.block_table),
                ctypes.c_int(meta.max_blocks), _ptr(meta.token_entry), _ptr(meta.positions), ctypes.c_int(S), ctypes.c_int(T),
-               ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(d), ctypes.c_float(scale), ctypes.c_int(win), _Hip.stream())
+               ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(d), ctypes.c_float(scale), ctypes.c_int(win), ctypes.c_float(softcap),
+               _Hip.stream())
     return out
 
 
@@ -1150,12 +1157,16 @@ def _row_view(x: torch.Tensor, what: str) -> int:
 
 
 def bias_rope_store(x: torch.Tensor, n_q: int, n_kv: int, d: int, bias: Optional[torch.Tensor], freq: Optional[torch.Tensor],
-                    rotary_dim: int, positions: torch.Tensor, k_cache, v_cache, page_size: int, slots: Optional[torch.Tensor]) -> torch.Tensor:
+                    rotary_dim: int, positions: torch.Tensor, k_cache, v_cache, page_size: int, slots: Optional[torch.Tensor],
+                    mag: float = 1.0, value_norm=None) -> torch.Tensor:
     """From rows ``x [T, >= (n_q + 2 n_kv) d]`` = [q heads | k heads | v heads] (a view into a wider product may be
     given): the biases ``bias [(n_q + 2 n_kv) d]`` added, the first ``rotary_dim`` dims of every q and k head rotated
     (pair (j, j + rotary_dim/2), angle float32(position) * freq[j]), q written to the result [T, n_q d], k and v into
-    the cache pages at ``slots`` (skipped when None)."""
+    the cache pages at ``slots`` (skipped when None).  ``mag``: factor on cos and sin.  ``value_norm`` = (eps, n): every
+    value head is divided by sqrt(mean of its first n values squared + eps) before it is stored."""
     xs = _row_view(x, "bias_rope_store")
+    v_eps, v_n = (float(value_norm[0]), int(value_norm[1])) if value_norm is not None else (0.0, 0)
+    _check(0 <= v_n <= d, "bias_rope_store: a value norm over %d of %d values", v_n, d)
     T = x.shape[0]
     _dev(bias, freq, positions, k_cache, v_cache, slots)
     _check(x.shape[1] >= (n_q + 2 * n_kv) * d, "bias_rope_store: rows of %d values hold no %d heads of %d", x.shape[1], n_q + 2 * n_kv, d)
@@ -1175,18 +1186,21 @@ def bias_rope_store(x: torch.Tensor, n_q: int, n_kv: int, d: int, bias: Optional
         hip().call("spy_bias_rope_store", ctypes.c_void_p(x.data_ptr()), ctypes.c_longlong(xs), _code(x, "x"), _ptr(q), ctypes.c_int(T),
                    ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(d), _ptr(bias), _code(bias, "bias") if bias is not None else F32,
                    _ptr(freq), ctypes.c_int(rotary_dim), _ptr(positions), _ptr(k_cache if slots is not None else None),
-                   _ptr(v_cache if slots is not None else None), ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(slots), _Hip.stream())
+                   _ptr(v_cache if slots is not None else None), ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(slots),
+                   ctypes.c_float(mag), ctypes.c_float(v_eps), ctypes.c_int(v_n), _Hip.stream())
     return q
 
 
-def sigmoid_gate(y: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
-    """In place: y[t, j] *= sigmoid(gate[t, j]); ``gate`` may be a view into a wider product."""
-    _dev(y)
+def sigmoid_gate(y: torch.Tensor, gate: torch.Tensor, bias: Optional[torch.Tensor] = None, mult: float = 1.0) -> torch.Tensor:
+    """In place: y[t, j] *= mult * sigmoid(gate[t, j] + bias[j]); ``gate`` may be a view into a wider product."""
+    _dev(y, bias)
+    _check(bias is None or bias.shape == (y.shape[1],), "sigmoid_gate: one bias per column expected")
     gs = _row_view(gate, "sigmoid_gate")
     _check(y.dim() == 2 and gate.shape == y.shape and gate.dtype == y.dtype and gate.device == y.device, "sigmoid_gate: gate rows like y expected")
     if y.numel():
-        hip().call("spy_sigmoid_gate", _ptr(y), ctypes.c_void_p(gate.data_ptr()), ctypes.c_longlong(gs), _code(y, "y"), ctypes.c_int(y.shape[0]),
-                   ctypes.c_int(y.shape[1]), _Hip.stream())
+        hip().call("spy_sigmoid_gate", _ptr(y), ctypes.c_void_p(gate.data_ptr()), ctypes.c_longlong(gs), _code(y, "y"), _ptr(bias),
+                   _code(bias, "bias") if bias is not None else F32, ctypes.c_float(mult), ctypes.c_int(y.shape[0]), ctypes.c_int(y.shape[1]),
+                   _Hip.stream())
     return y
 
 
@@ -1276,13 +1290,14 @@ def causal_conv_silu(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, k
 
 def delta_rule(qkv: torch.Tensor, beta_pre: torch.Tensor, dec_pre: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
                gate: torch.Tensor, norm_w: torch.Tensor, eps: float, state: torch.Tensor, cu_q: torch.Tensor, slot_ids: torch.Tensor,
-               H: int, G: int, d: int, dv: int) -> torch.Tensor:
+               H: int, G: int, d: int, dv: int, gate_act: str = "sigmoid") -> torch.Tensor:
     """The gated delta rule over the step's tokens.  ``qkv [T, 2 G d + H dv]``: q and k (G heads of d; made unit vectors
     here, q also times d^-1/2) and v (H heads of dv); ``beta_pre [T, H]`` and ``dec_pre [T, H d]`` float32: the raw products
     (overwritten with what they turn into) behind beta = sigmoid(.) and the decay exp(-exp(a_log[h]) softplus(. + dt_bias)) per head and key channel; per head
     S = diag(decay) S, u = beta (v - S^T k), S += k u^T, o = S^T q with ``state[slot, h d dv ..]`` float32.  Returns
     [T, H dv]: o over its root mean square, times ``norm_w [dv]``, times sigmoid(``gate``) (rows of H dv values, a view
-    into a wider product allowed)."""
+    into a wider product allowed; ``gate_act`` "silu": times silu(gate)).  One decay per head instead of one per key
+    channel: ``dec_pre [T, H]`` and ``dt_bias [H]``."""
     _dev(qkv, beta_pre, dec_pre, a_log, dt_bias, norm_w, state, cu_q, slot_ids)
     gs = _row_view(gate, "delta_rule")
     T = qkv.shape[0]
@@ -1291,10 +1306,12 @@ def delta_rule(qkv: torch.Tensor, beta_pre: torch.Tensor, dec_pre: torch.Tensor,
            "delta_rule: qkv [T, 2 G d + H dv] and gate rows [T, H dv] of one dtype expected")
     _check(H % G == 0 and 0 < d <= MATRIX_MEMORY_MAX_DIM and 0 < dv <= MATRIX_MEMORY_MAX_VDIM, "delta_rule: heads of %d x %d (up to %d x %d)",
            d, dv, MATRIX_MEMORY_MAX_DIM, MATRIX_MEMORY_MAX_VDIM)
-    _check(beta_pre.dtype == torch.float32 and beta_pre.shape == (T, H) and dec_pre.dtype == torch.float32 and dec_pre.shape == (T, H * d),
-           "delta_rule: the products behind beta [T, H] and the decay [T, H d] must be float32")
-    _check(a_log.shape == (H,) and dt_bias.shape == (H * d,) and norm_w.shape == (dv,) and a_log.dtype == dt_bias.dtype == norm_w.dtype,
-           "delta_rule: a_log [H], dt_bias [H d] and a norm weight [dv] of one dtype expected")
+    dd = 1 if dec_pre.dim() == 2 and dec_pre.shape[1] == H and dt_bias.shape == (H,) else d        # decays per head: one, or one per key channel
+    _check(gate_act in ("sigmoid", "silu"), "delta_rule: the gate's activation is sigmoid or silu")
+    _check(beta_pre.dtype == torch.float32 and beta_pre.shape == (T, H) and dec_pre.dtype == torch.float32 and dec_pre.shape == (T, H * dd),
+           "delta_rule: the products behind beta [T, H] and the decay [T, H d] (or [T, H]) must be float32")
+    _check(a_log.shape == (H,) and dt_bias.shape == (H * dd,) and norm_w.shape == (dv,) and a_log.dtype == dt_bias.dtype == norm_w.dtype,
+           "delta_rule: a_log [H], dt_bias [H d] (or [H]) and a norm weight [dv] of one dtype expected")
     _check(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= H * d * dv, "delta_rule: state must be float32 [slots, >= H d dv]")
     out = torch.empty((T, H * dv), dtype=qkv.dtype, device=qkv.device)
     if T:
@@ -1303,18 +1320,89 @@ def delta_rule(qkv: torch.Tensor, beta_pre: torch.Tensor, dec_pre: torch.Tensor,
         hip().call("spy_delta_rule", _ptr(out), _ptr(tmp), _ptr(unit), _ptr(state), ctypes.c_longlong(state.shape[1]), _ptr(qkv), _code(qkv, "qkv"), _ptr(beta_pre),
                    _ptr(dec_pre), _ptr(a_log), _ptr(dt_bias), _code(a_log, "decay numbers"), ctypes.c_void_p(gate.data_ptr()), ctypes.c_longlong(gs),
                    _ptr(norm_w), ctypes.c_float(eps), _ptr(cu_q), _ptr(slot_ids), ctypes.c_int(state.shape[0]), ctypes.c_int(S), ctypes.c_int(T),
-                   ctypes.c_int(H), ctypes.c_int(G), ctypes.c_int(d), ctypes.c_int(dv), _Hip.stream())
+                   ctypes.c_int(H), ctypes.c_int(G), ctypes.c_int(d), ctypes.c_int(dv), ctypes.c_int(dd), ctypes.c_int(1 if gate_act == "silu" else 0),
+                   _Hip.stream())
+    return out
+
+
+def token_shift(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, keep_off: int, token_entry: torch.Tensor, cu_q: torch.Tensor,
+                slot_ids: torch.Tensor) -> torch.Tensor:
+    """out[s, t, c] = x[t, c] + (x'[t, c] - x[t, c]) mu[s, c], x' the row of the token before t in its request: the
+    entry's row before, or, for an entry's first token, the request's kept row ``state[slot, keep_off + c]`` (float32;
+    zeros for a request's first token), which afterwards holds the entry's last row.  ``mu [n, W]`` -> [n, T, W]."""
+    _dev(x, mu, state, token_entry, cu_q, slot_ids)
+    _check(x.dim() == 2 and x.dtype in _CODES and mu.dim() == 2 and mu.shape[1] == x.shape[1], "token_shift: rows [T, W] and blends [n, W] expected")
+    T, W = x.shape
+    S = _entries(cu_q, slot_ids, "token_shift")
+    _check(token_entry.dtype == torch.int32 and token_entry.shape == (T,), "token_shift: token_entry must be int32 [T]")
+    _check(state.dtype == torch.float32 and state.dim() == 2 and 0 <= keep_off and keep_off + W <= state.shape[1],
+           "token_shift: the kept row reaches beyond the float32 state")
+    out = torch.empty((mu.shape[0], T, W), dtype=x.dtype, device=x.device)
+    if T:
+        hip().call("spy_token_shift", _ptr(out), _ptr(x), _code(x, "x"), _ptr(mu), _code(mu, "blends"), ctypes.c_int(mu.shape[0]),
+                   ctypes.c_void_p(state.data_ptr() + 4 * keep_off), ctypes.c_longlong(state.shape[1]), _ptr(token_entry), _ptr(cu_q),
+                   _ptr(slot_ids), ctypes.c_int(state.shape[0]), ctypes.c_int(S), ctypes.c_int(T), ctypes.c_int(W), _Hip.stream())
+    return out
+
+
+def tanh_(x: torch.Tensor) -> torch.Tensor:
+    """tanh in place over a float32 tensor."""
+    _dev(x)
+    _check(x.dtype == torch.float32, "tanh_: float32 expected")
+    if x.numel():
+        hip().call("spy_tanh", _ptr(x), ctypes.c_longlong(x.numel()), _Hip.stream())
+    return x
+
+
+def time_mix(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, dec_pre: torch.Tensor, w0: torch.Tensor, u: torch.Tensor, gate: torch.Tensor,
+             norm_w: torch.Tensor, eps: float, state: torch.Tensor, cu_q: torch.Tensor, slot_ids: torch.Tensor, H: int, d: int) -> torch.Tensor:
+    """Per head a state S [d, d] (``state[slot, h d d ..]`` float32, row = key channel): o = (S + diag(u) k v^T)^T r, then
+    S = diag(w) S + k v^T with w = exp(-exp(dec_pre + w0)) per key channel.  ``r``, ``k``, ``v``, ``gate [T, H d]``;
+    ``dec_pre [T, H d]`` float32 (overwritten with the decays); ``w0``, ``u``, ``norm_w [H d]``.  Returns [T, H d]: each head's
+    o over its root mean square, times ``norm_w``, times silu(gate)."""
+    _dev(r, k, v, dec_pre, w0, u, gate, norm_w, state, cu_q, slot_ids)
+    T, N = r.shape
+    S = _entries(cu_q, slot_ids, "time_mix")
+    _check(N == H * d and 0 < d <= MATRIX_MEMORY_MAX_DIM, "time_mix: %d heads of %d (up to %d)", H, d, MATRIX_MEMORY_MAX_DIM)
+    _check(r.dtype in _CODES and all(t.shape == (T, N) and t.dtype == r.dtype for t in (k, v, gate)), "time_mix: r, k, v and gate [T, H d] of one dtype expected")
+    _check(dec_pre.dtype == torch.float32 and dec_pre.shape == (T, N), "time_mix: the decay's products must be float32 [T, H d]")
+    _check(all(t.shape == (N,) for t in (w0, u, norm_w)) and w0.dtype == u.dtype == norm_w.dtype, "time_mix: w0, u and a norm weight [H d] of one dtype expected")
+    _check(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= H * d * d, "time_mix: state must be float32 [slots, >= H d d]")
+    out = torch.empty((T, N), dtype=r.dtype, device=r.device)
+    if T:
+        tmp = torch.empty((T, N), dtype=torch.float32, device=r.device)           # the read-outs before the heads' norm
+        bonus = torch.empty((T, H), dtype=torch.float32, device=r.device)         # sum_i r u k per token and head
+        hip().call("spy_time_mix", _ptr(out), _ptr(tmp), _ptr(bonus), _ptr(state), ctypes.c_longlong(state.shape[1]), _ptr(r), _ptr(k), _ptr(v),
+                   _ptr(gate), _code(r, "r"), _ptr(dec_pre), _ptr(w0), _ptr(u), _ptr(norm_w), _code(w0, "decay numbers"), ctypes.c_float(eps),
+                   _ptr(cu_q), _ptr(slot_ids), ctypes.c_int(state.shape[0]), ctypes.c_int(S), ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(d),
+                   _Hip.stream())
+    return out
+
+
+def norm_pair_mean(a: torch.Tensor, b: torch.Tensor, wa: torch.Tensor, wb: torch.Tensor, eps: float) -> torch.Tensor:
+    """(a / rms(a) * wa + b / rms(b) * wb) / 2 per row, float32 inside; the result has the rows' dtype."""
+    _dev(a, b, wa, wb)
+    _check(a.dim() == 2 and a.shape == b.shape and a.dtype == b.dtype and a.dtype in _CODES, "norm_pair_mean: two sets of rows of one shape and dtype expected")
+    T, W = a.shape
+    _check(wa.shape == (W,) and wb.shape == (W,) and wa.dtype == wb.dtype, "norm_pair_mean: weights [W] of one dtype expected")
+    out = torch.empty_like(a)
+    if T:
+        hip().call("spy_norm_pair_mean", _ptr(out), _ptr(a), _ptr(b), _code(a, "rows"), _ptr(wa), _ptr(wb), _code(wa, "norm weight"),
+                   ctypes.c_float(eps), ctypes.c_int(T), ctypes.c_int(W), _Hip.stream())
     return out
 
 
 # --------------------------------------------------------------------------
 # Mixture of experts
-def moe_route(z: torch.Tensor, correction: torch.Tensor, top: int, groups: int, keep: int, scale: float):
-    """Router logits ``z [T, E]`` float32 -> (experts int32 [T, top], weights float32 [T, top]): s = softmax(z); the choice
-    goes by s + ``correction`` among the experts of the ``keep`` best of ``groups`` equal groups of neighbours (a group's
-    score: its largest choice score); the weights are the chosen s over their sum (+ 1e-20), times ``scale``."""
+def moe_route(z: torch.Tensor, correction: Optional[torch.Tensor], top: int, groups: int, keep: int, scale: float, score: str = "softmax",
+              renormalize: bool = True):
+    """Router logits ``z [T, E]`` float32 -> (experts int32 [T, top], weights float32 [T, top]): s = softmax(z) (``score``
+    "sigmoid": sigmoid of each logit); the choice goes by s + ``correction`` (None: by s) among the experts of the ``keep``
+    best of ``groups`` equal groups of neighbours (a group's score: its largest choice score); the weights are the chosen s
+    over their sum (+ 1e-20; ``renormalize`` False: as they are), times ``scale``."""
     _dev(z, correction)
-    _check(z.dtype == torch.float32 and z.dim() == 2 and correction.dtype == torch.float32 and correction.shape == (z.shape[1],),
+    _check(score in ("softmax", "sigmoid"), "moe_route: scores are softmax or sigmoid")
+    _check(z.dtype == torch.float32 and z.dim() == 2 and (correction is None or (correction.dtype == torch.float32 and correction.shape == (z.shape[1],))),
            "moe_route: logits float32 [T, E] and a float32 correction [E] expected")
     T, E = z.shape
     _check(0 < groups and E % groups == 0 and 0 < keep <= groups and 0 < top <= keep * (E // groups) and E <= 1024,
@@ -1323,17 +1411,24 @@ def moe_route(z: torch.Tensor, correction: torch.Tensor, top: int, groups: int, 
     w = torch.empty((T, top), dtype=torch.float32, device=z.device)
     if T:
         hip().call("spy_moe_route", _ptr(ids), _ptr(w), _ptr(z), _ptr(correction), ctypes.c_int(T), ctypes.c_int(E), ctypes.c_int(top),
-                   ctypes.c_int(groups), ctypes.c_int(keep), ctypes.c_float(scale), _Hip.stream())
+                   ctypes.c_int(groups), ctypes.c_int(keep), ctypes.c_float(scale), ctypes.c_int(1 if score == "sigmoid" else 0),
+                   ctypes.c_int(1 if renormalize else 0), _Hip.stream())
     return ids, w
 
 
 MOE_MFMA = True            # False forces the plain float32 kernel for bfloat16 too (tests flip it; nothing else does)
 
 
-def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
+def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
+                activation: str = "silu", limit: float = 0.0, weight_input: bool = False) -> torch.Tensor:
     """out[t] = sum_k weights[t, k] * down_e( silu(gate_e x[t]) * up_e x[t] ), e = ids[t, k]; ``w_gate_up [E, 2 F, K]`` =
     every expert's [gate rows | up rows], ``w_down [E, K, F]``.  The (token, choice) pairs are sorted by expert on the
-    device and the experts' products run over the sorted rows; no size here depends on the choice."""
+    device and the experts' products run over the sorted rows; no size here depends on the choice.  ``activation``
+    "clamped": g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(1.702 g) (u + 1) in place of silu(gate) up.
+    ``weight_input``: the weight multiplies the expert's input, out[t] = sum_k expert_e(weights[t, k] x[t]) (the two
+    products being linear, it is multiplied into their sums, ahead of the activation)."""
+    _check(activation in ("silu", "clamped") and (activation == "silu" or limit > 0.0), "moe_experts: activation silu, or clamped with a positive limit")
+    act_kind = 1 if activation == "clamped" else 0
     _dev(x, ids, weights, w_gate_up, w_down)
     T, K = x.shape
     top = ids.shape[1]
@@ -1361,12 +1456,12 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
     act = torch.empty((max_tiles * tm, F), dtype=x.dtype, device=dev)
     hip().call("spy_moe_gemm", _ptr(act), _code(act, "act"), _ptr(x), _code(x, "x"), _ptr(w_gate_up), _code(w_gate_up, "expert matrices"),
                _ptr(tile_expert), _ptr(sorted_pair), ctypes.c_int(top), ctypes.c_int(1), ctypes.c_int(max_tiles), ctypes.c_int(E), ctypes.c_int(F),
-               ctypes.c_int(K), ctypes.c_int(per_block), _Hip.stream())
+               ctypes.c_int(K), ctypes.c_int(per_block), ctypes.c_int(act_kind), ctypes.c_float(limit), _ptr(weights if weight_input else None), _Hip.stream())
     y = torch.empty((max_tiles * tm, K), dtype=torch.float32, device=dev)
     hip().call("spy_moe_gemm", _ptr(y), F32, _ptr(act), _code(act, "act"), _ptr(w_down), _code(w_down, "expert matrices"), _ptr(tile_expert),
                _ptr(sorted_pair), ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(max_tiles), ctypes.c_int(E), ctypes.c_int(K), ctypes.c_int(F),
-               ctypes.c_int(per_block), _Hip.stream())
-    hip().call("spy_moe_combine", _ptr(out), _code(out, "out"), _ptr(y), _ptr(weights), _ptr(pair_row), ctypes.c_int(T), ctypes.c_int(top),
+               ctypes.c_int(per_block), ctypes.c_int(0), ctypes.c_float(0.0), _ptr(None), _Hip.stream())
+    hip().call("spy_moe_combine", _ptr(out), _code(out, "out"), _ptr(y), _ptr(None if weight_input else weights), _ptr(pair_row), ctypes.c_int(T), ctypes.c_int(top),
                ctypes.c_int(K), _Hip.stream())
     return out
 

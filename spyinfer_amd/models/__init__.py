@@ -1,4 +1,5 @@
 from . import qwen3  # registers "Qwen3ForCausalLM"
 from . import sefevik  # registers "Sefevik"
 from . import sodedra  # registers "Sodedra"
+from . import meronex  # registers "Meronex"
 from .base import DecoderModel, LayerCall

@@ -67,23 +67,35 @@ class DecoderModel:
 
     # ---- cache -----------------------------------------------------------
     def cache_specs(self) -> List[Optional[object]]:
-        """Need of every cache id, taken from the call that writes it."""
+        """Need of every cache id, taken from the call that writes it.  A mixer made of several (its ``cache_spec`` is a
+        list) has the call's cache id for the first of them and further ids, behind the calls' own, for the others; its
+        ``forward`` is handed the layer caches as a tuple in the list's order."""
         ids = [c.cache for c in self.schedule if c.cache is not None]
         specs: List[Optional[object]] = [None] * (max(ids) + 1 if ids else 0)
-        writers = {}
+        writers, several = {}, {}
         for call in self.schedule:
             if call.cache is None or not call.store:
                 continue
             if call.cache in writers:
                 raise ValueError("cache %d is written by two calls of the run order" % call.cache)
             writers[call.cache] = call
-            specs[call.cache] = self.layers[call.layer].mixer.cache_spec()
+            need = self.layers[call.layer].mixer.cache_spec()
+            if isinstance(need, (list, tuple)):
+                several[call.cache] = list(need)
+                need = need[0] if need else None
+            specs[call.cache] = need
         for call in self.schedule:
             if call.cache is not None and not call.store:
                 if call.cache not in writers:
                     raise ValueError("a call reads cache %d that no call writes" % call.cache)
-                if self.layers[call.layer].mixer.cache_spec() != specs[call.cache]:
+                need = self.layers[call.layer].mixer.cache_spec()
+                if (list(need) != several.get(call.cache)) if isinstance(need, (list, tuple)) else (call.cache in several or need != specs[call.cache]):
                     raise ValueError("layer %d reads cache %d of another shape" % (call.layer, call.cache))
+        #: cache id of a call -> the ids of all caches of its mixer, for mixers made of several
+        self.cache_parts = {}
+        for cid in sorted(several):
+            self.cache_parts[cid] = [cid] + list(range(len(specs), len(specs) + len(several[cid]) - 1))
+            specs += several[cid][1:]
         # an embedding that keeps something per request (the token before, say) has the cache id after the layers'
         own = getattr(self.embed, "cache_spec", None)
         self.embed_cache = None
@@ -127,6 +139,8 @@ class DecoderModel:
             resid, pending = self.position.on_embeddings(self.embed.forward(batch.token_ids), batch), None
         for i, call in enumerate(calls):
             cache = storage.layer(call.cache) if call.cache is not None else None
+            if call.cache in self.cache_parts:
+                cache = tuple(storage.layer(c) for c in self.cache_parts[call.cache])
             resid, pending = self.layers[call.layer].forward(resid, pending, batch, cache, call.store, next_norm=entry[i + 1])
         if batch.R == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=resid.device) if logits_out is None else logits_out

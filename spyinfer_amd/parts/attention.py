@@ -13,7 +13,8 @@ Options beside the reference's arrangement: biases on the q, k and v projections
 key size (the smaller of the two is padded with zero rows when the weights are bound, so that one head size runs
 through cache and kernels); a sigmoid gate on the concatenated heads, projected from the mixer's input beside
 q, k and v; a rotation whose angles are formed in the kernel from the encoding's frequencies (no table and no
-position limit: encodings with rescaled frequencies).
+position limit: encodings with rescaled frequencies, with or without a factor on cos and sin); values divided by their
+root mean square per head before they are stored; scores capped by cap tanh(score / cap) after the scale.
 """
 from __future__ import annotations
 
@@ -102,12 +103,14 @@ class PagedAttention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: Optional[PositionEncoding], qk_norm_eps: Optional[float] = None,
                  window: Optional[int] = None, scale: Optional[float] = None, fold_rows: Optional[int] = None,
-                 value_dim: Optional[int] = None, bias: bool = False, gate: bool = False, names: Optional[dict] = None):
+                 value_dim: Optional[int] = None, bias: bool = False, gate: bool = False, names: Optional[dict] = None,
+                 softcap: float = 0.0, value_norm_eps: Optional[float] = None):
         """``fold_rows``: most rows of a step whose products here run with the norms and the residual sum folded in
         (None: ``ops.default_fold_rows`` of this part's matrices).  ``value_dim``: size of a value head (None: ``head_dim``).
         ``bias``: q, k and v have biases.  ``gate``: the heads' results are multiplied by sigmoid(Wg x) before the output
         projection.  ``names``: tensor names behind the prefix for q, k, v, o, g, q_norm, k_norm and the biases' suffix
-        ``bias``."""
+        ``bias``.  ``softcap`` > 0: score = softcap tanh(q . k scale / softcap).  ``value_norm_eps``: every value head is
+        divided by sqrt(mean(v^2) + eps) over its ``value_dim`` values (no weight) and cached so."""
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
         self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
@@ -124,6 +127,8 @@ class PagedAttention(Mixer):
         self.window = window
         self.scale = 1.0 / math.sqrt(head_dim) if scale is None else float(scale)
         self.fold_rows = fold_rows
+        self.softcap = float(softcap or 0.0)
+        self.value_norm_eps = None if value_norm_eps is None else float(value_norm_eps)
         self.w_qkv = self.w_o = self.q_norm = self.k_norm = self.w_qkv_tiled = self.w_o_tiled = None
 
     # ---- weights ---------------------------------------------------------
@@ -202,7 +207,8 @@ class PagedAttention(Mixer):
         """No bias, no gate and a rotation by table: the arrangement that the fused kernels and the folded products know.
         Otherwise one kernel adds the biases, rotates by angles that it forms itself from the encoding's frequencies (an
         encoding with rescaled frequencies has no table) and stores."""
-        return not (self.has_bias or self.has_gate or (self.position is not None and getattr(self.position, "scaling", None) is not None))
+        return not (self.has_bias or self.has_gate or self.softcap or self.value_norm_eps is not None
+                    or (self.position is not None and getattr(self.position, "scaling", None) is not None))
 
     def _rotated_whole(self) -> bool:
         """The head is rotated whole or not at all, and the group is one tile: what the fused kernel takes."""
@@ -250,14 +256,14 @@ class PagedAttention(Mixer):
             # which lie behind them, are multiplied into the heads' results
             if self.qk_norm_eps is not None:
                 raise ValueError("per-head norms of q and k beside biases, a gate or rescaled frequencies are not implemented")
-            freq, rdim = None, 0
+            freq, mag, rdim = None, 1.0, 0
             if self.position is not None:
                 freq, mag, rdim = self.position.frequencies()
-                if mag != 1.0:
-                    raise ValueError("a factor on cos and sin is not implemented for this attention")
             slots = batch.slot_mapping(cache.group) if store else None
-            q = ops.bias_rope_store(qkv, nq, nkv, d, self.b_qkv, freq, rdim, batch.positions, cache.k, cache.v, cache.page_size, slots)
-            out = ops.paged_attention(q, cache.k, cache.v, cache.page_size, meta, nq, nkv, d, self.scale, self.window)
+            vnorm = None if self.value_norm_eps is None else (self.value_norm_eps, self.value_dim)
+            q = ops.bias_rope_store(qkv, nq, nkv, d, self.b_qkv, freq, rdim, batch.positions, cache.k, cache.v, cache.page_size, slots,
+                                    mag=mag, value_norm=vnorm)
+            out = ops.paged_attention(q, cache.k, cache.v, cache.page_size, meta, nq, nkv, d, self.scale, self.window, softcap=self.softcap)
             if self.has_gate:
                 ops.sigmoid_gate(out, qkv[:, (nq + 2 * nkv) * d:])
             return out

@@ -9,14 +9,47 @@ from ..weights.loader import WeightSpec
 from .base import Block, FeedForward, Mixer, Norm, Part
 
 
+class ResultGate(Part):
+    """What a sublayer's result is multiplied by before it meets the stream: ``mult`` * sigmoid(W n + b), element by
+    element, n being the sublayer's input (the norm's output).  Tensors: the matrix under the prefix itself, the bias
+    under ``<prefix>.b``."""
+
+    def __init__(self, hidden_size: int, mult: float = 1.0, bias_suffix: str = ".b"):
+        self.hidden_size, self.mult, self.bias_suffix = hidden_size, float(mult), bias_suffix
+        self.w = self.w_tiled = self.bias = None
+
+    def weight_specs(self, prefix):
+        H = self.hidden_size
+        return [WeightSpec(prefix, (H, H)), WeightSpec(prefix + self.bias_suffix, (H,), "bias")]
+
+    def bind(self, prefix, weights):
+        self.w, self.w_tiled = ops.weight_forms(weights.pop(prefix))
+        self.bias = weights[prefix + self.bias_suffix]
+
+    def capturable(self, batch):
+        return True
+
+    def apply(self, y, n):
+        """y * mult * sigmoid(W n + b), in place over y."""
+        return ops.sigmoid_gate(y, ops.linear_few(n, self.w, self.w_tiled), self.bias, self.mult)
+
+
 class PreNormBlock(Block):
-    def __init__(self, norm1: Norm, mixer: Mixer, norm2: Norm, ffn: FeedForward,
-                 names=("input_layernorm", "self_attn", "post_attention_layernorm", "mlp")):
+    def __init__(self, norm1: Norm, mixer: Mixer, norm2: Norm = None, ffn: FeedForward = None,
+                 names=("input_layernorm", "self_attn", "post_attention_layernorm", "mlp"), gates=None, gate_names=("rg1", "rg2")):
+        """``ffn`` (with ``norm2``) may be absent.  ``gates``: None, or a pair of ``ResultGate`` (the second None without a
+        feed-forward) that multiply the two sublayers' results, each reading its sublayer's input."""
+        if (ffn is None) != (norm2 is None):
+            raise ValueError("a feed-forward and its norm come together")
         self.norm1, self.mixer, self.norm2, self.ffn = norm1, mixer, norm2, ffn
         self.names = names
+        self.gate1, self.gate2 = gates if gates is not None else (None, None)
+        self.gate_names = gate_names
 
     def _parts(self, prefix):
-        return zip((self.norm1, self.mixer, self.norm2, self.ffn), (prefix + "." + n for n in self.names))
+        parts = list(zip((self.norm1, self.mixer, self.norm2, self.ffn), (prefix + "." + n for n in self.names)))
+        parts += list(zip((self.gate1, self.gate2), (prefix + "." + n for n in self.gate_names)))
+        return [(part, p) for part, p in parts if part is not None]
 
     def weight_specs(self, prefix):
         return [s for part, p in self._parts(prefix) for s in part.weight_specs(p)]
@@ -29,13 +62,14 @@ class PreNormBlock(Block):
         return self.norm1
 
     def capturable(self, batch):
-        return all(part.capturable(batch) for part in (self.norm1, self.mixer, self.norm2, self.ffn))
+        return all(part.capturable(batch) for part, _ in self._parts(""))
 
     def forward(self, resid, pending, batch, cache, store=True, next_norm=None):
         act = batch.act_dtype
         ready = isinstance(pending, ops.ScaledInput)
         mine = ready and pending.norm is self.norm1
-        fold = self.norm2.foldable(act) is not None and self.mixer.can_fold(batch) and self.ffn.can_fold(batch)
+        plain = self.ffn is not None and self.gate1 is None and self.gate2 is None
+        fold = plain and self.norm2.foldable(act) is not None and self.mixer.can_fold(batch) and self.ffn.can_fold(batch)
         if fold and not ops.folded_products_take(pending if mine else None, batch.T):
             # beyond 64 rows the folded products take an input in operand order only, which only the part before this
             # block can have prepared (another kind of block, a position encoding on the embeddings, parts that fold up
@@ -53,8 +87,13 @@ class PreNormBlock(Block):
             return resid, self.ffn.forward(n2, batch)
         n1 = self.norm1.add_norm(resid, None if ready else pending, act)
         a = self.mixer.forward(n1, batch, cache, store)
+        if self.gate1 is not None:
+            a = self.gate1.apply(a, n1)
+        if self.ffn is None:
+            return resid, a
         n2 = self.norm2.add_norm(resid, a, act)
-        return resid, self.ffn.forward(n2, batch)
+        f = self.ffn.forward(n2, batch)
+        return resid, (self.gate2.apply(f, n2) if self.gate2 is not None else f)
 
 
 def stream_copy(batch, resid, copy=None):

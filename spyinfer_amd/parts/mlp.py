@@ -98,7 +98,19 @@ class MoEMLP(FeedForward):
     ``e<i>.down``."""
 
     def __init__(self, hidden_size: int, expert_size: int, experts: int, top: int, groups: int = 1, groups_kept: int = 1,
-                 scale: float = 1.0, names=("router", "correction", "e%d.gate", "e%d.up", "e%d.down")):
+                 scale: float = 1.0, names=("router", "correction", "e%d.gate", "e%d.up", "e%d.down"), score: str = "softmax",
+                 renormalize: bool = True, correction: bool = True, weight_on: str = "output", activation: str = "silu",
+                 limit: float = 0.0):
+        """``score``: "softmax" over all experts or "sigmoid" of each logit.  ``renormalize``: the chosen scores over their
+        sum (else as they are), times ``scale``.  ``correction``: a stored vector is added to the scores for the choice.
+        ``weight_on``: "output": out = sum w expert(x); "input": out = sum expert(w x).  ``activation``: "silu":
+        silu(gate) * up; "clamped": g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(1.702 g) (u + 1)."""
+        if score not in ("softmax", "sigmoid") or weight_on not in ("output", "input") or activation not in ("silu", "clamped"):
+            raise ValueError("MoEMLP: score %r, weight_on %r or activation %r is not implemented" % (score, weight_on, activation))
+        if activation == "clamped" and not limit > 0.0:
+            raise ValueError("MoEMLP: the clamped activation needs a positive limit")
+        self.score, self.renormalize, self.has_correction, self.weight_on = score, bool(renormalize), bool(correction), weight_on
+        self.activation, self.limit = activation, float(limit)
         if experts <= 0 or groups <= 0 or experts % groups or not 0 < groups_kept <= groups or not 0 < top <= groups_kept * (experts // groups):
             raise ValueError("a choice of %d among %d of %d groups of %d experts cannot be made" % (top, groups_kept, groups, experts))
         self.hidden_size, self.expert_size, self.experts, self.top = hidden_size, expert_size, experts, top
@@ -108,7 +120,7 @@ class MoEMLP(FeedForward):
     def weight_specs(self, prefix):
         H, F, E = self.hidden_size, self.expert_size, self.experts
         router, corr, gate, up, down = (prefix + "." + n for n in self.names)
-        specs = [WeightSpec(router, (E, H)), WeightSpec(corr, (E,), "bias")]
+        specs = [WeightSpec(router, (E, H))] + ([WeightSpec(corr, (E,), "bias")] if self.has_correction else [])
         for e in range(E):
             specs += [WeightSpec(gate % e, (F, H)), WeightSpec(up % e, (F, H)), WeightSpec(down % e, (H, F))]
         return specs
@@ -118,7 +130,7 @@ class MoEMLP(FeedForward):
         # the router's product keeps its float32 sums (bfloat16 operands multiply exactly in float32), and everything
         # behind it is float32: its scores decide, they are not activations
         self.w_router = weights.pop(router)
-        self.correction = weights[corr].float().contiguous()
+        self.correction = weights[corr].float().contiguous() if self.has_correction else None
         E = self.experts
         mats = [weights.pop(n % e) for e in range(E) for n in (gate, up, down)]
         if len({m.dtype for m in mats}) > 1:
@@ -132,5 +144,7 @@ class MoEMLP(FeedForward):
 
     def forward(self, x, batch):
         z = ops.linear(x, self.w_router, torch.float32)
-        ids, weights = ops.moe_route(z, self.correction, self.top, self.groups, self.groups_kept, self.scale)
-        return ops.moe_experts(x, ids, weights, self.w_gate_up, self.w_down)
+        ids, weights = ops.moe_route(z, self.correction, self.top, self.groups, self.groups_kept, self.scale, score=self.score,
+                                     renormalize=self.renormalize)
+        return ops.moe_experts(x, ids, weights, self.w_gate_up, self.w_down, activation=self.activation, limit=self.limit,
+                               weight_input=self.weight_on == "input")

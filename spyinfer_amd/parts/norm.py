@@ -11,14 +11,18 @@ from .base import Norm
 
 
 class RMSNorm(Norm):
-    def __init__(self, size: int, eps: float, suffix: str = ".weight", offset: float = 0.0):
-        """``suffix``: what the weight's name has behind the part's prefix (some checkpoints name the vector by the
+    def __init__(self, size: int, eps: float, suffix: str = ".weight", offset: float = 0.0, groups: int = 1):
+        """``groups``: the vector is cut into that many equal consecutive parts, each over its own root mean square (the
+        weight still spans the whole vector).  ``suffix``: what the weight's name has behind the part's prefix (some checkpoints name the vector by the
         prefix alone).  ``offset``: the stored vector is centred on zero and multiplies as ``offset + w`` (1.0 for norms
         whose weights are stored around zero); the sum is formed once, in float32, when the weights are bound."""
         self.size = size
         self.eps = float(eps)
         self.suffix = suffix
         self.offset = float(offset)
+        self.groups = int(groups)
+        if self.groups <= 0 or size % self.groups:
+            raise ValueError("a norm in %d groups does not fit a vector of %d" % (self.groups, size))
         self.weight = None
 
     def weight_specs(self, prefix):
@@ -37,19 +41,21 @@ class RMSNorm(Norm):
         """``delta``: None, one addend, or a pair of addends (the results of two sublayers that read the same norm)."""
         if isinstance(delta, (tuple, list)):
             first, second = delta
-            return ops.add_rms_norm(resid, first, self.weight, self.eps, out_dtype, rows, delta2=second)
-        return ops.add_rms_norm(resid, delta, self.weight, self.eps, out_dtype, rows)
+            return ops.add_rms_norm(resid, first, self.weight, self.eps, out_dtype, rows, delta2=second, groups=self.groups)
+        return ops.add_rms_norm(resid, delta, self.weight, self.eps, out_dtype, rows, groups=self.groups)
 
     def add_normed(self, base, y, out=None, copy_dtype=None, mix=None):
         """out = base + norm(y) in float32 (the norm on a sublayer's output; ``out`` may be ``base``); returns (out, its
         copy in ``copy_dtype`` or None).  ``mix`` = (kept results [layers, T, H], n, weights [n]) with ``out`` the n-th
         kept result: the weighted sum of the n results is formed in the same pass and returned in place of ``out``."""
+        if self.groups != 1:
+            raise ValueError("a norm in groups on a sublayer's output is not implemented")
         if mix is not None and mix[2].dtype != self.weight.dtype:
             out, _ = ops.norm_residual(base, y, self.weight, self.eps, out, None)
             return ops.depth_mix(mix[0], mix[1], mix[2], copy_dtype)
         return ops.norm_residual(base, y, self.weight, self.eps, out, copy_dtype, mix)
 
     def foldable(self, out_dtype):
-        if out_dtype == torch.bfloat16 and self.weight is not None and self.weight.dtype == torch.bfloat16:
+        if self.groups == 1 and out_dtype == torch.bfloat16 and self.weight is not None and self.weight.dtype == torch.bfloat16:
             return self.weight, self.eps
         return None

@@ -15,6 +15,15 @@ short causal convolution per channel and silu, q and k become unit vectors (q al
 S = diag(g) S with a decay g = exp(-exp(A_h) softplus(W2 W1 x + bias)) per head and key channel; u = beta (v - S^T k),
 beta = sigmoid(Wb x); S += k u^T; o = S^T q; each head's o over its root mean square, times a weight shared by the
 heads, times sigmoid(G2 G1 x), then the output projection.  The convolutions' last inputs are state of the request too.
+``HeadDelta``: the same rule with ONE decay per head, g = exp(-exp(A_h) softplus(Wa x + bias_h)), and the output gate
+silu(Wg x) from a full projection.
+
+``TimeMix``: a state S [key size, key size] per head with a decay per key channel, read BEFORE the token's write except
+for the token's own contribution, which enters through a learned bonus u:  o = (S + diag(u) k v^T)^T r;
+S = diag(w) S + k v^T.  Every projection reads its own blend of the token's input and the input of the token before it,
+x + (x' - x) mu (x' = 0 for a request's first token); w = exp(-exp(W2 tanh(W1 blend_w) + w0)); each head's o over its
+root mean square, times a weight, times silu(Wg blend_g), then the output projection.  The input of a request's last
+token is state of the request too.
 """
 from __future__ import annotations
 
@@ -240,3 +249,128 @@ class ChannelDelta(Mixer):
         y = ops.delta_rule(qkv, beta_pre, dec_pre, self.a_log, self.dt_bias, gate, self.norm, self.norm_eps, cache.state, cu_q, slots,
                            H, G, d, dv)
         return ops.linear_few(y, self.w_o, self.w_o_tiled)
+
+
+class HeadDelta(Mixer):
+    """The gated delta rule with one decay per head and a full output gate (see the module's text)."""
+
+    def __init__(self, hidden_size: int, heads: int, kv_heads: int, dim: int, vdim: int, conv: int, norm_eps: float,
+                 names=("q", "k", "v", "b", "a", "g", "o", "q.conv", "k.conv", "v.conv", "A_log", "dt_bias", "norm")):
+        if heads % kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        if not 1 <= conv <= 8:
+            raise ValueError("the short convolution has 1 to 8 taps")
+        self.hidden_size, self.heads, self.kv_heads, self.dim, self.vdim, self.conv = hidden_size, heads, kv_heads, dim, vdim, conv
+        self.norm_eps, self.names = float(norm_eps), names
+        self.w_in = self.w_in_tiled = self.w_small = self.w_o = self.w_o_tiled = None
+        self.taps = self.a_log = self.dt_bias = self.norm = None
+
+    def _channels(self):
+        return 2 * self.kv_heads * self.dim + self.heads * self.vdim
+
+    def weight_specs(self, prefix):
+        W, H, G, d, dv, n = self.hidden_size, self.heads, self.kv_heads, self.dim, self.vdim, self.conv
+        q, k, v, b, a, g, o, qc, kc, vc, alog, dtb, norm = (prefix + "." + x for x in self.names)
+        return [WeightSpec(q, (G * d, W)), WeightSpec(k, (G * d, W)), WeightSpec(v, (H * dv, W)), WeightSpec(b, (H, W)),
+                WeightSpec(a, (H, W)), WeightSpec(g, (H * dv, W)), WeightSpec(o, (W, H * dv)), WeightSpec(qc, (G * d, n), "bias"),
+                WeightSpec(kc, (G * d, n), "bias"), WeightSpec(vc, (H * dv, n), "bias"), WeightSpec(alog, (H,), "bias"),
+                WeightSpec(dtb, (H,), "bias"), WeightSpec(norm, (dv,), "norm")]
+
+    def bind(self, prefix, weights):
+        q, k, v, b, a, g, o, qc, kc, vc, alog, dtb, norm = (prefix + "." + x for x in self.names)
+        mats = [weights.pop(n) for n in (q, k, v, g)]
+        if len({m.dtype for m in mats}) > 1:
+            mats = [m.float() for m in mats]
+        # one product for the wide projections: rows [q | k | v | gate]; what enters the recurrence's exponentials (beta,
+        # the decay) comes from a second, small product that stays float32
+        self.w_in, self.w_in_tiled = ops.weight_forms(torch.cat(mats, dim=0).contiguous())
+        del mats
+        small = [weights.pop(b), weights.pop(a)]
+        if small[0].dtype != small[1].dtype:
+            small = [t.float() for t in small]
+        self.w_small = torch.cat(small, dim=0).contiguous()
+        self.w_o, self.w_o_tiled = ops.weight_forms(weights.pop(o))
+        taps = [weights[n] for n in (qc, kc, vc)]
+        vecs = [weights[alog], weights[dtb], weights[norm]]
+        if len({t.dtype for t in taps + vecs}) > 1:
+            taps, vecs = [t.float() for t in taps], [t.float() for t in vecs]
+        self.taps = torch.cat(taps, dim=0).contiguous()
+        self.a_log, self.dt_bias, self.norm = vecs
+
+    def cache_spec(self):
+        H, d, dv = self.heads, self.dim, self.vdim
+        return FixedState((H * d * dv + (self.conv - 1) * self._channels(),), "float32")
+
+    def capturable(self, batch):
+        return True
+
+    def forward(self, x, batch, cache, store=True):
+        if not store:
+            raise ValueError("a recurrence cannot run on another layer's state without writing it")
+        H, G, d, dv, C = self.heads, self.kv_heads, self.dim, self.vdim, self._channels()
+        proj = ops.linear_few(x, self.w_in, self.w_in_tiled)
+        small = ops.linear(x, self.w_small, torch.float32)                    # [beta | decay], float32 sums kept
+        beta_pre, dec_pre = small[:, :H].contiguous(), small[:, H:].contiguous()
+        cu_q, slots = batch.array("cu_q"), batch.array("slot_ids")
+        qkv = ops.causal_conv_silu(proj[:, :C], self.taps, cache.state, H * d * dv, batch.array("token_entry"), cu_q, slots)
+        y = ops.delta_rule(qkv, beta_pre, dec_pre, self.a_log, self.dt_bias, proj[:, C:], self.norm, self.norm_eps, cache.state, cu_q, slots,
+                           H, G, d, dv, gate_act="silu")
+        return ops.linear_few(y, self.w_o, self.w_o_tiled)
+
+
+class TimeMix(Mixer):
+    """Token shift and a per-head state with a decay per key channel and a bonus for the current token (see the module's
+    text).  Tensors: ``mu.r/k/v/g/w [W]``, ``r``, ``k``, ``v``, ``g [H d, W]``, ``w1 [rank, W]``, ``w2 [H d, rank]``,
+    ``w0 [H d]``, ``u [H, d]``, ``norm [H d]``, ``o [W, H d]``; the decay's inner size is the stored tensors'."""
+
+    BLENDS = ("r", "k", "v", "g", "w")
+
+    def __init__(self, hidden_size: int, heads: int, dim: int, norm_eps: float, decay_rank: int = None,
+                 names=("mu.%s", "r", "k", "v", "g", "w1", "w2", "w0", "u", "norm", "o")):
+        self.hidden_size, self.heads, self.dim, self.norm_eps, self.names = hidden_size, heads, dim, float(norm_eps), names
+        self.rank = -1 if decay_rank is None else decay_rank
+        self.mu = self.w_r = self.w_k = self.w_v = self.w_g = self.w_1 = self.w_2 = self.w_o = None
+        self.w0 = self.u = self.norm = None
+
+    def weight_specs(self, prefix):
+        W, N = self.hidden_size, self.heads * self.dim
+        mu, r, k, v, g, w1, w2, w0, u, norm, o = (prefix + "." + x for x in self.names)
+        specs = [WeightSpec(mu % b, (W,), "mix") for b in self.BLENDS]
+        specs += [WeightSpec(n, (N, W)) for n in (r, k, v, g)]
+        specs += [WeightSpec(w1, (self.rank, W)), WeightSpec(w2, (N, self.rank)), WeightSpec(w0, (N,), "bias"),
+                  WeightSpec(u, (self.heads, self.dim), "bias"), WeightSpec(norm, (N,), "norm"), WeightSpec(o, (W, N))]
+        return specs
+
+    def bind(self, prefix, weights):
+        mu, r, k, v, g, w1, w2, w0, u, norm, o = (prefix + "." + x for x in self.names)
+        if weights[w2].shape[1] != weights[w1].shape[0]:
+            raise ValueError("%s: the inner sizes of the decay's two projections do not fit each other" % prefix)
+        mus = [weights[mu % b] for b in self.BLENDS]
+        vecs = [weights[w0], weights[u].reshape(-1), weights[norm]]
+        if len({t.dtype for t in mus + vecs}) > 1:
+            mus, vecs = [t.float() for t in mus], [t.float() for t in vecs]
+        self.mu = torch.stack(mus).contiguous()
+        self.w0, self.u, self.norm = (t.contiguous() for t in vecs)
+        self.w_r, self.w_k, self.w_v, self.w_g = (ops.weight_forms(weights.pop(n)) for n in (r, k, v, g))
+        # the decay's two products keep their float32 sums: what they give enters two exponentials
+        self.w_1, self.w_2 = weights.pop(w1), weights.pop(w2)
+        self.w_o = ops.weight_forms(weights.pop(o))
+
+    def cache_spec(self):
+        return FixedState((self.heads * self.dim * self.dim + self.hidden_size,), "float32")
+
+    def capturable(self, batch):
+        return True
+
+    def forward(self, x, batch, cache, store=True):
+        if not store:
+            raise ValueError("a recurrence cannot run on another layer's state without writing it")
+        H, d = self.heads, self.dim
+        cu_q, slots = batch.array("cu_q"), batch.array("slot_ids")
+        blends = ops.token_shift(x, self.mu, cache.state, H * d * d, batch.array("token_entry"), cu_q, slots)      # [5, T, W]
+        r, k, v, g = (ops.linear_few(blends[i], w[0], w[1]) for i, w in enumerate((self.w_r, self.w_k, self.w_v, self.w_g)))
+        inner = ops.tanh_(ops.linear(blends[4], self.w_1, torch.float32))
+        # (the inner projection's result is an activation: it takes the activation dtype on its way into the outer one)
+        dec_pre = ops.linear(inner.to(self.w_2.dtype).contiguous(), self.w_2, torch.float32)
+        y = ops.time_mix(r, k, v, dec_pre, self.w0, self.u, g, self.norm, self.norm_eps, cache.state, cu_q, slots, H, d)
+        return ops.linear_few(y, self.w_o[0], self.w_o[1])

@@ -11,7 +11,7 @@ class EmuOps:
     def embedding(self, ids, table, scale=1.0):
         return table[ids.long()].float() * scale
 
-    def add_rms_norm(self, resid, delta, weight, eps, out_dtype, rows=None, delta2=None):
+    def add_rms_norm(self, resid, delta, weight, eps, out_dtype, rows=None, delta2=None, groups=1):
         if delta is not None and delta2 is not None:
             delta = delta.float() + delta2.float()
         if rows is None:
@@ -22,8 +22,9 @@ class EmuOps:
             x = resid[rows.long()]
             if delta is not None:
                 x = x + delta[rows.long()].float()
-        r = torch.rsqrt((x * x).mean(dim=-1, keepdim=True) + eps)
-        return (x * r * weight.float()).to(out_dtype)
+        xg = x.reshape(x.shape[0], groups, -1)
+        r = torch.rsqrt((xg * xg).mean(dim=-1, keepdim=True) + eps)
+        return ((xg * r).reshape(x.shape) * weight.float()).to(out_dtype)
 
     def rms_norm(self, x, weight, eps):
         xf = x.float()
@@ -62,7 +63,7 @@ class EmuOps:
                 v_cache[page, :, :, off] = v[t].to(v_cache.dtype)
         return q.reshape(T, n_q * d).to(qkv.dtype)
 
-    def paged_attention(self, q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window):
+    def paged_attention(self, q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window, softcap=0.0):
         T = meta.T
         out = torch.zeros((T, n_q, d), dtype=torch.float32)
         qf = q.float().reshape(T, n_q, d)
@@ -80,6 +81,8 @@ class EmuOps:
             for h in range(n_q):
                 g = h * n_kv // n_q
                 sc = (K[:, g, :] @ qf[t, h]) * scale
+                if softcap:
+                    sc = softcap * torch.tanh(sc / softcap)
                 pr = torch.softmax(sc, dim=0)
                 out[t, h] = pr @ V[:, g, :]
         return out.reshape(T, n_q * d).to(q.dtype)
@@ -217,7 +220,8 @@ class EmuOps:
         return out.to(out_dtype)
 
     # ---- attention with biases, angles formed per call, an output gate ----
-    def bias_rope_store(self, x, n_q, n_kv, d, bias, freq, rotary_dim, positions, k_cache, v_cache, page_size, slots):
+    def bias_rope_store(self, x, n_q, n_kv, d, bias, freq, rotary_dim, positions, k_cache, v_cache, page_size, slots, mag=1.0,
+                        value_norm=None):
         T = x.shape[0]
         n = (n_q + 2 * n_kv) * d
         f = x[:, :n].float()
@@ -227,7 +231,10 @@ class EmuOps:
         k = f[:, n_q * d:(n_q + n_kv) * d].reshape(T, n_kv, d)
         v = f[:, (n_q + n_kv) * d:].reshape(T, n_kv, d)
         if rotary_dim:
-            q, k = self._rotate(q, positions, freq, 1.0, rotary_dim), self._rotate(k, positions, freq, 1.0, rotary_dim)
+            q, k = self._rotate(q, positions, freq, mag, rotary_dim), self._rotate(k, positions, freq, mag, rotary_dim)
+        if value_norm is not None:
+            eps, n = value_norm
+            v = v * torch.rsqrt((v[..., :n] ** 2).mean(-1, keepdim=True) + eps)
         if slots is not None:
             for t in range(T):
                 sl = int(slots[t])
@@ -237,8 +244,9 @@ class EmuOps:
                 v_cache[sl // page_size, :, :, sl % page_size] = v[t].to(v_cache.dtype)
         return q.reshape(T, n_q * d).to(x.dtype)
 
-    def sigmoid_gate(self, y, gate):
-        y.copy_((y.float() * torch.sigmoid(gate.float())).to(y.dtype))
+    def sigmoid_gate(self, y, gate, bias=None, mult=1.0):
+        g = gate.float() if bias is None else gate.float() + bias.float()
+        y.copy_((y.float() * torch.sigmoid(g) * mult).to(y.dtype))
         return y
 
     # ---- matrix memories ----
@@ -287,7 +295,7 @@ class EmuOps:
                 keep.copy_(rows[rows.shape[0] - (n - 1):])
         return y.to(x.dtype)
 
-    def delta_rule(self, qkv, beta_pre, dec_pre, a_log, dt_bias, gate, norm_w, eps, state, cu_q, slot_ids, H, G, d, dv):
+    def delta_rule(self, qkv, beta_pre, dec_pre, a_log, dt_bias, gate, norm_w, eps, state, cu_q, slot_ids, H, G, d, dv, gate_act="sigmoid"):
         T = qkv.shape[0]
         f = qkv.float()
         q = f[:, :G * d].reshape(T, G, d)
@@ -296,7 +304,8 @@ class EmuOps:
         q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * d ** -0.5
         k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
         beta = torch.sigmoid(beta_pre)
-        dec = torch.exp(-torch.exp(a_log.float())[None, :, None] * torch.nn.functional.softplus(dec_pre + dt_bias.float()).view(T, H, d))
+        dec = torch.exp(-torch.exp(a_log.float())[None, :, None] * torch.nn.functional.softplus(dec_pre + dt_bias.float()).view(T, H, -1))
+        dec = dec.expand(T, H, d)              # (one decay per head: the same for all its key channels)
         out = torch.zeros((T, H, dv), dtype=torch.float32)
         for s in range(slot_ids.shape[0]):
             st = state[int(slot_ids[s]), :H * d * dv].view(H, d, dv)
@@ -310,26 +319,67 @@ class EmuOps:
                     out[t, h] = S.T @ q[t, g]
                 st[h] = S
         out = out * torch.rsqrt((out * out).mean(-1, keepdim=True) + eps) * norm_w.float()
-        return (out.reshape(T, H * dv) * torch.sigmoid(gate.float())).to(qkv.dtype)
+        g = gate.float()
+        return (out.reshape(T, H * dv) * (torch.sigmoid(g) if gate_act == "sigmoid" else g * torch.sigmoid(g))).to(qkv.dtype)
+
+    # ---- token shift and the state with a decay per key channel ----
+    def token_shift(self, x, mu, state, keep_off, token_entry, cu_q, slot_ids):
+        T, W = x.shape
+        f = x.float()
+        prev = torch.zeros_like(f)
+        for s in range(slot_ids.shape[0]):
+            keep = state[int(slot_ids[s]), keep_off:keep_off + W]
+            t0, t1 = int(cu_q[s]), int(cu_q[s + 1])
+            prev[t0] = keep
+            prev[t0 + 1:t1] = f[t0:t1 - 1]
+            keep.copy_(f[t1 - 1])
+        return (f[None] + (prev - f)[None] * mu.float()[:, None, :]).to(x.dtype)
+
+    def tanh_(self, x):
+        return x.copy_(torch.tanh(x))
+
+    def time_mix(self, r, k, v, dec_pre, w0, u, gate, norm_w, eps, state, cu_q, slot_ids, H, d):
+        T = r.shape[0]
+        rf, kf, vf = (t.float().reshape(T, H, d) for t in (r, k, v))
+        dec = torch.exp(-torch.exp(dec_pre + w0.float())).view(T, H, d)
+        uu = u.float().view(H, d)
+        out = torch.zeros((T, H, d), dtype=torch.float32)
+        for s in range(slot_ids.shape[0]):
+            st = state[int(slot_ids[s]), :H * d * d].view(H, d, d)
+            S = st.clone()
+            for t in range(int(cu_q[s]), int(cu_q[s + 1])):
+                kv = kf[t][:, :, None] * vf[t][:, None, :]
+                out[t] = torch.einsum("hi,hij->hj", rf[t], S + uu[:, :, None] * kv)
+                S = dec[t][:, :, None] * S + kv
+            st.copy_(S)
+        out = out * torch.rsqrt((out * out).mean(-1, keepdim=True) + eps)
+        g = gate.float()
+        return (out.reshape(T, H * d) * norm_w.float() * g * torch.sigmoid(g)).to(r.dtype)
+
+    def norm_pair_mean(self, a, b, wa, wb, eps):
+        af, bf = a.float(), b.float()
+        na = af * torch.rsqrt((af * af).mean(-1, keepdim=True) + eps) * wa.float()
+        nb = bf * torch.rsqrt((bf * bf).mean(-1, keepdim=True) + eps) * wb.float()
+        return (0.5 * (na + nb)).to(a.dtype)
 
     # ---- mixture of experts ----
-    def moe_route(self, z, correction, top, groups, keep, scale):
+    def moe_route(self, z, correction, top, groups, keep, scale, score="softmax", renormalize=True):
         T, E = z.shape
         per = E // groups
         ids = torch.zeros((T, top), dtype=torch.int32)
         w = torch.zeros((T, top), dtype=torch.float32)
         for t in range(T):
-            s = torch.softmax(z[t].float(), dim=0)
-            ch = (s + correction.float()).tolist()
+            s = torch.softmax(z[t].float(), dim=0) if score == "softmax" else torch.sigmoid(z[t].float())
+            ch = (s + correction.float()).tolist() if correction is not None else s.tolist()
             best = sorted(range(groups), key=lambda g: (-max(ch[g * per:(g + 1) * per]), g))[:keep]
             allowed = [e for e in range(E) if e // per in best]
             chosen = sorted(allowed, key=lambda e: (-ch[e], e))[:top]
-            tot = sum(float(s[e]) for e in chosen) + 1e-20
+            tot = (sum(float(s[e]) for e in chosen) + 1e-20) if renormalize else 1.0
             for j, e in enumerate(chosen):
                 ids[t, j], w[t, j] = e, float(s[e]) / tot * scale
         return ids, w
 
-    def moe_experts(self, x, ids, weights, w_gate_up, w_down):
+    def moe_experts(self, x, ids, weights, w_gate_up, w_down, activation="silu", limit=0.0, weight_input=False):
         T, K = x.shape
         F = w_gate_up.shape[1] // 2
         out = torch.zeros((T, K), dtype=torch.float32)
@@ -338,6 +388,13 @@ class EmuOps:
             for j in range(ids.shape[1]):
                 e = int(ids[t, j])
                 gu = w_gate_up[e].float() @ xf[t]
-                act = (gu[:F] * torch.sigmoid(gu[:F]) * gu[F:]).to(x.dtype).float()
-                out[t] += weights[t, j] * (w_down[e].float() @ act)
+                if weight_input:
+                    gu = gu * weights[t, j]
+                if activation == "silu":
+                    act = gu[:F] * torch.sigmoid(gu[:F]) * gu[F:]
+                else:
+                    g, u = torch.clamp(gu[:F], max=limit), torch.clamp(gu[F:], -limit, limit)
+                    act = g * torch.sigmoid(1.702 * g) * (u + 1.0)
+                act = act.to(x.dtype).float()
+                out[t] += (1.0 if weight_input else weights[t, j]) * (w_down[e].float() @ act)
         return out.to(x.dtype)
