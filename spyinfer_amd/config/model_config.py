@@ -477,6 +477,8 @@ class MeronexConfig(ModelConfig):
             right = _need(m, "right", dict, at)
             mix = {"left": cls._attention(_need(m, "left", dict, at), at + ".left"),
                    "right": {k: _need(right, k, int, at + ".right") for k in ("heads", "dim")}}
+            # the inner size of the decay's two projections: no key of the design; the stored tensors decide unless it is given
+            mix["right"]["decay_rank"] = _need(right, "decay_rank", int, at + ".right") if right.get("decay_rank") is not None else None
         out = {"type": kind, "mixer": mix, "mlp": None}
         mlp = raw.get("mlp")
         if mlp is not None:

@@ -32,7 +32,7 @@ def build_meronex(cfg: MeronexConfig) -> DecoderModel:
             position = RotaryEmbedding(a["dim"], rot["base"], rot["dims"], rot["scaling"]) if rot else None
             left = PagedAttention(W, a["heads"], a["kv_heads"], a["dim"], position, scale=a["scale"], value_dim=a["vdim"],
                                   names=ATTENTION_NAMES, softcap=a["softcap"], value_norm_eps=eps)
-            mixer = SideBySide(W, left, TimeMix(W, t["heads"], t["dim"], eps), eps)
+            mixer = SideBySide(W, left, TimeMix(W, t["heads"], t["dim"], eps, t["decay_rank"]), eps)
         f = layer["mlp"]
         ffn = None
         if f is not None:

@@ -335,7 +335,7 @@ class TimeMix(Mixer):
     def weight_specs(self, prefix):
         W, N = self.hidden_size, self.heads * self.dim
         mu, r, k, v, g, w1, w2, w0, u, norm, o = (prefix + "." + x for x in self.names)
-        specs = [WeightSpec(mu % b, (W,), "mix") for b in self.BLENDS]
+        specs = [WeightSpec(mu % b, (W,), "bias") for b in self.BLENDS]
         specs += [WeightSpec(n, (N, W)) for n in (r, k, v, g)]
         specs += [WeightSpec(w1, (self.rank, W)), WeightSpec(w2, (N, self.rank)), WeightSpec(w0, (N,), "bias"),
                   WeightSpec(u, (self.heads, self.dim), "bias"), WeightSpec(norm, (N,), "norm"), WeightSpec(o, (W, N))]
