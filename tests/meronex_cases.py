@@ -120,6 +120,15 @@ def long_memory(forget_bias=6.0, a_log=-4.0, w0=-5.0):
     return tweak
 
 
+def decisive_router(factor=4.0):
+    """Router logits spread out, so that fewer choices hang on a difference of the size of a bfloat16 rounding."""
+    def tweak(tensors):
+        for name in tensors:
+            if name.endswith(".mlp.router"):
+                tensors[name] = (tensors[name].float() * factor).to(tensors[name].dtype)
+    return tweak
+
+
 def both(*tweaks):
     def tweak(tensors):
         for t in tweaks:
