@@ -23,6 +23,7 @@ Other workloads, each again one JSON line:
     python bench.py --shape 32b --batch 64 --prompt-len 4096 --context 4608 --points "" --steps 32 --warmup 4   # long keys at the 32B shape
     python bench.py --design sefevik [--design-sizes 1024,2048,4096] [--layers 8]   # Sefevik beside Qwen3 at equal size
     python bench.py --design sodedra [--design-sizes 1024,2048,4096] [--layers 8]   # Sodedra beside Qwen3 at equal size
+    python bench.py --design meronex [--design-sizes 1024,2048,4096] [--layers 9]   # Meronex beside Sodedra and Qwen3 at equal size
 """
 import argparse
 import json
@@ -96,7 +97,31 @@ def sodedra_shape(width: int, layers: int, vocab: int, window: int = 1024) -> di
     return dict(architecture="Sodedra", vocab=vocab, width=width, norm=dict(eps=1e-6), embedding=dict(scale=1.0), layers=out)
 
 
-DESIGN_SHAPES = {"sefevik": ("Sefevik", sefevik_shape), "sodedra": ("Sodedra", sodedra_shape)}
+def meronex_shape(width: int, layers: int, vocab: int) -> dict:
+    """A Meronex configuration with the layer sizes of a real model of that width: of every three layers an mLSTM (keys
+    of 128, values of 256, half as many heads), a delta rule with one decay per head (heads of 128 x 128, half as many q/k
+    heads, 4 taps) and an attention (heads of 128 with 64 rotated dims, a quarter as many kv heads, capped scores) beside
+    a time mix (heads of 64, a decay of inner size 64); every feed-forward 32 experts of 3/4 width of which a token uses
+    four (as many active weights as a dense layer of three times the width); norms in 4 groups."""
+    heads = max(1, width // 128)
+    rot = dict(base=500000.0, dims=64, scaling=dict(factor=8.0, original=8192, fast=32.0, slow=1.0))
+    left = dict(heads=heads, kv_heads=max(1, heads // 4), dim=128, vdim=128, scale=128 ** -0.5, softcap=50.0, rot=rot)
+    moe = dict(kind="moe", expert=dict(ff=3 * width // 4, limit=7.0), router=dict(experts=32, top=4))
+    out = []
+    for i in range(layers):
+        kind = i % 3
+        if kind == 0:
+            out.append(dict(type="mlstm", mixer=dict(heads=max(1, heads // 2), dim=128, vdim=256, gate_cap=16.0), mlp=moe))
+        elif kind == 1:
+            out.append(dict(type="delta", mixer=dict(heads=heads, kv_heads=max(1, heads // 2), dim=128, vdim=128, conv=4), mlp=moe))
+        else:
+            out.append(dict(type="parallel", mixer=dict(left=dict(left), right=dict(heads=max(1, width // 64), dim=64, decay_rank=64)), mlp=moe))
+    return dict(architecture="Meronex", vocab=vocab, width=width, norm=dict(eps=1e-6, groups=4), residual_mult=0.5, layers=out)
+
+
+DESIGN_SHAPES = {"sefevik": ("Sefevik", sefevik_shape), "sodedra": ("Sodedra", sodedra_shape), "meronex": ("Meronex", meronex_shape)}
+#: further designs that a design is measured beside (Qwen3 always is): the closest one the engine has
+DESIGN_BESIDE = {"meronex": ("sodedra",)}
 
 
 def design_compare(args) -> int:
@@ -121,9 +146,10 @@ def design_compare(args) -> int:
     results = {}
     for width in [int(x) for x in args.design_sizes.split(",") if x.strip()]:
         heads = max(1, width // 128)
-        raws = {design: shape_of(width, layers, vocab),
-                "qwen3": dict(MODEL_8B, num_hidden_layers=layers, hidden_size=width, num_attention_heads=heads,
-                              num_key_value_heads=max(1, heads // 4), intermediate_size=3 * width, vocab_size=vocab)}
+        raws = {design: shape_of(width, layers, vocab)}
+        raws.update({other: DESIGN_SHAPES[other][1](width, layers, vocab) for other in DESIGN_BESIDE.get(design, ())})
+        raws.update({"qwen3": dict(MODEL_8B, num_hidden_layers=layers, hidden_size=width, num_attention_heads=heads,
+                              num_key_value_heads=max(1, heads // 4), intermediate_size=3 * width, vocab_size=vocab)})
         for name, raw in raws.items():
             arch = architecture_of(raw)
             cfg = arch.config_cls.from_dict(raw)
@@ -209,7 +235,7 @@ def main() -> int:
     ap.add_argument("--serve", type=int, default=0, metavar="N",
                     help="instead of the decode steps: N requests arriving at once, prompts of 128..2048 and outputs of 64..512 "
                          "tokens (uniform), run until all have ended; the value is generated tokens per second of the whole run")
-    ap.add_argument("--design", default="", choices=["", "sefevik", "sodedra"],
+    ap.add_argument("--design", default="", choices=["", "sefevik", "sodedra", "meronex"],
                     help="instead of the decode steps: prefill and decode throughput of that design at a few layer sizes "
                          "beside the Qwen3 shape of equal width, layers, heads and feed-forward size (--design-sizes)")
     ap.add_argument("--design-sizes", default="1024,2048,4096", help="widths for --design")

@@ -130,7 +130,9 @@ template <> struct Vec4<bf16_t> {
 template <typename TA, typename TW, bool VEC>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restrict__ delta, const TA* __restrict__ delta2,
                                    const TW* __restrict__ w, float eps, TA* __restrict__ out, const int* __restrict__ rows, int T,
-                                   int H, int ld) {
+                                   int H, int ld, const TA* __restrict__ gate, const TW* __restrict__ gbias, float mult) {
+    // gate != null: the addend is delta * mult * sigmoid(gate + gbias), element by element (a sublayer's result behind its
+    // gate), formed here in float32 from the sublayer's result and the gate's product.
     // H: values that are normed together: the whole row (ld == H), or one of the row's ld / H consecutive groups, which
     // blockIdx.y counts
     __shared__ float red[16];
@@ -148,6 +150,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
     const TA* dl = delta ? delta + (size_t)t * ld + g0 : nullptr;
     const TA* dl2 = delta2 ? delta2 + (size_t)t * ld + g0 : nullptr;
     TA* o = out + (size_t)r * ld + g0;
+    const TA* gt = gate ? gate + (size_t)t * ld + g0 : nullptr;
+    const TW* gb = gate ? gbias + g0 : nullptr;
     w += g0;
     const bool write_back = dl && !rows;
     if (VEC) {
@@ -167,6 +171,13 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
                         Vec4<TA>::load(dl2 + i, e4);
 #pragma unroll
                         for (int e = 0; e < 4; ++e) d4[e] += e4[e];
+                    }
+                    if (gt) {
+                        float g4[4], b4[4];
+                        Vec4<TA>::load(gt + i, g4);
+                        Vec4<TW>::load(gb + i, b4);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) d4[e] = d4[e] * mult / (1.0f + expf(-(g4[e] + b4[e])));
                     }
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[p][e] += d4[e];
@@ -194,7 +205,11 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
     float ss = 0.f;
     for (int i = threadIdx.x; i < H; i += blockDim.x) {
         float v = x[i];
-        if (dl) v += to_f32<TA>(dl[i]) + (dl2 ? to_f32<TA>(dl2[i]) : 0.f);
+        if (dl) {
+            float a = to_f32<TA>(dl[i]) + (dl2 ? to_f32<TA>(dl2[i]) : 0.f);
+            if (gt) a = a * mult / (1.0f + expf(-(to_f32<TA>(gt[i]) + to_f32<TW>(gb[i]))));
+            v += a;
+        }
         if (write_back) x[i] = v;
         ss += v * v;
     }
@@ -202,28 +217,34 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
     const float scale = 1.0f / sqrtf(ss / (float)H + eps);
     for (int i = threadIdx.x; i < H; i += blockDim.x) {
         float v = x[i];
-        if (dl && rows) v += to_f32<TA>(dl[i]) + (dl2 ? to_f32<TA>(dl2[i]) : 0.f);
+        if (dl && rows) {
+            float a = to_f32<TA>(dl[i]) + (dl2 ? to_f32<TA>(dl2[i]) : 0.f);
+            if (gt) a = a * mult / (1.0f + expf(-(to_f32<TA>(gt[i]) + to_f32<TW>(gb[i]))));
+            v += a;
+        }
         o[i] = from_f32<TA>((scale * v) * to_f32<TW>(w[i]));
     }
 }
 
 extern "C" int spy_add_rmsnorm(float* resid, const void* delta, const void* delta2, const void* w, int w_dtype, float eps, void* out,
-                               int out_dtype, const int* rows, int n_out, int T, int ld, int groups, hipStream_t st) {
+                               int out_dtype, const int* rows, int n_out, int T, int ld, int groups, const void* gate, const void* gbias,
+                               float mult, hipStream_t st) {
     SPY_REQUIRE(n_out > 0 && T > 0 && ld > 0, "spy_add_rmsnorm: empty operand");
+    SPY_REQUIRE(!gate || (delta && gbias), "spy_add_rmsnorm: a gate without an addend or without its bias");
     SPY_REQUIRE(groups > 0 && groups <= 65535 && ld % groups == 0, "spy_add_rmsnorm: %d groups do not divide rows of %d", groups, ld);
     SPY_REQUIRE(delta || !delta2, "spy_add_rmsnorm: a second addend without a first");
     const int H = ld / groups;
     const dim3 grid(n_out, groups);
     const int threads = H >= 2048 ? 256 : (H >= 512 ? 128 : 64);
     const bool aligned = H % 4 == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)delta % 16) == 0 && ((uintptr_t)delta2 % 16) == 0 && ((uintptr_t)w % 16) == 0 &&
-                         ((uintptr_t)out % 16) == 0;
+                         ((uintptr_t)out % 16) == 0 && ((uintptr_t)gate % 16) == 0 && ((uintptr_t)gbias % 16) == 0;
     const bool vec = aligned && H <= threads * 4 * NORM_PASSES;
     if (vec) {
         SPY_DISPATCH(out_dtype, TA, SPY_DISPATCH(w_dtype, TW, (add_rmsnorm_kernel<TA, TW, true><<<grid, threads, 0, st>>>(
-            resid, (const TA*)delta, (const TA*)delta2, (const TW*)w, eps, (TA*)out, rows, T, H, ld))));
+            resid, (const TA*)delta, (const TA*)delta2, (const TW*)w, eps, (TA*)out, rows, T, H, ld, (const TA*)gate, (const TW*)gbias, mult))));
     } else {
         SPY_DISPATCH(out_dtype, TA, SPY_DISPATCH(w_dtype, TW, (add_rmsnorm_kernel<TA, TW, false><<<grid, 512, 0, st>>>(
-            resid, (const TA*)delta, (const TA*)delta2, (const TW*)w, eps, (TA*)out, rows, T, H, ld))));
+            resid, (const TA*)delta, (const TA*)delta2, (const TW*)w, eps, (TA*)out, rows, T, H, ld, (const TA*)gate, (const TW*)gbias, mult))));
     }
     SPY_CHECK_LAUNCH("spy_add_rmsnorm");
     return 0;

@@ -137,10 +137,12 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> tor
 
 
 def add_rms_norm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
-                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None, delta2: Optional[torch.Tensor] = None, groups: int = 1) -> torch.Tensor:
+                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None, delta2: Optional[torch.Tensor] = None, groups: int = 1,
+                 gate=None) -> torch.Tensor:
     """resid += delta (float32, in place; skipped if delta is None), then RMS-normalise.  ``delta2``: a second addend
     (two sublayers that read one norm): resid += delta + delta2, the two summed in float32 first.  ``groups``: the row is
-    cut into that many equal consecutive parts, each over its own root mean square.
+    cut into that many equal consecutive parts, each over its own root mean square.  ``gate`` = (rows [T, H] of the activation
+    dtype, bias [H] of the weight's dtype, constant): the addend is delta * constant * sigmoid(rows + bias), formed in float32.
 
     Without ``rows``: every row is updated and normalised -> [T, H].  With ``rows``
     (int32 [R]): only those rows are summed and normalised -> [R, H]; resid is left as it is."""
@@ -155,12 +157,17 @@ def add_rms_norm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: tor
         _check(delta.shape == (T, H) and delta.dtype == out_dtype, "add_rms_norm: delta must be [T, H] of the activation dtype")
     if rows is not None:
         _check(rows.dtype == torch.int32 and rows.dim() == 1, "add_rms_norm: rows must be int32 [R]")
+    g_rows, g_bias, g_mult = gate if gate is not None else (None, None, 1.0)
+    if gate is not None:
+        _dev(g_rows, g_bias)
+        _check(delta is not None and g_rows.shape == (T, H) and g_rows.dtype == out_dtype and g_bias.shape == (H,) and g_bias.dtype == weight.dtype,
+               "add_rms_norm: the gate's rows must be like the addend and its bias like the norm's weight")
     n_out = T if rows is None else rows.shape[0]
     out = torch.empty((n_out, H), dtype=out_dtype, device=resid.device)
     if n_out:
         hip().call("spy_add_rmsnorm", _ptr(resid), _ptr(delta), _ptr(delta2), _ptr(weight), _code(weight, "norm weight"),
                    ctypes.c_float(eps), _ptr(out), _code(out, "norm output"), _ptr(rows), ctypes.c_int(n_out),
-                   ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(groups), _Hip.stream())
+                   ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(groups), _ptr(g_rows), _ptr(g_bias), ctypes.c_float(g_mult), _Hip.stream())
     return out
 
 
@@ -397,6 +404,18 @@ class OperandRows:
         """The same values as an ordinary [M, K] tensor (for tests; not used by the engine)."""
         mt = self.tiles
         return self.data.view(self.width // 32, mt, 4, 16, 8).permute(1, 3, 0, 2, 4).reshape(16 * mt, self.width)[:self.rows].contiguous()
+
+
+class GatedAddend:
+    """A sublayer's result that meets the stream behind a gate: the addend is ``y * mult * sigmoid(gate + bias)``.  The
+    norm that sums it into the stream forms it in the same pass (``add_rms_norm(gate=)``); whoever cannot calls ``resolve``."""
+    __slots__ = ("y", "gate", "bias", "mult")
+
+    def __init__(self, y, gate, bias, mult):
+        self.y, self.gate, self.bias, self.mult = y, gate, bias, mult
+
+    def resolve(self):
+        return sigmoid_gate(self.y, self.gate, self.bias, self.mult)
 
 
 class ScaledInput:

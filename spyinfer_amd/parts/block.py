@@ -30,8 +30,8 @@ class ResultGate(Part):
         return True
 
     def apply(self, y, n):
-        """y * mult * sigmoid(W n + b), in place over y."""
-        return ops.sigmoid_gate(y, ops.linear_few(n, self.w, self.w_tiled), self.bias, self.mult)
+        """y * mult * sigmoid(W n + b) as an addend whose gate the next norm's kernel applies (``ops.GatedAddend``)."""
+        return ops.GatedAddend(y, ops.linear_few(n, self.w, self.w_tiled), self.bias, self.mult)
 
 
 class PreNormBlock(Block):
@@ -185,7 +185,7 @@ class OutputNormBlock(Block):
         act = batch.act_dtype
         if pending is not None and not isinstance(pending, ops.ScaledInput):
             for addend in (pending if isinstance(pending, (tuple, list)) else (pending,)):
-                resid.add_(addend.float())         # a block of another arrangement left an addend (or a pair of them)
+                resid.add_((addend.resolve() if isinstance(addend, ops.GatedAddend) else addend).float())         # a block of another arrangement left an addend (or a pair of them)
         x = stream_copy(batch, resid)
         y = self.mixer.forward(x, batch, cache, store)
         out = self.depth.result_slot(batch, resid) if self.depth is not None else resid

@@ -39,6 +39,13 @@ class RMSNorm(Norm):
 
     def add_norm(self, resid, delta, out_dtype, rows=None):
         """``delta``: None, one addend, or a pair of addends (the results of two sublayers that read the same norm)."""
+        if isinstance(delta, ops.GatedAddend):
+            # a sublayer's result behind its gate: formed in this kernel's pass where the dtypes allow it
+            if delta.bias.dtype != self.weight.dtype or not delta.gate.is_contiguous():
+                delta = delta.resolve()
+            else:
+                return ops.add_rms_norm(resid, delta.y, self.weight, self.eps, out_dtype, rows, groups=self.groups,
+                                        gate=(delta.gate, delta.bias, delta.mult))
         if isinstance(delta, (tuple, list)):
             first, second = delta
             return ops.add_rms_norm(resid, first, self.weight, self.eps, out_dtype, rows, delta2=second, groups=self.groups)

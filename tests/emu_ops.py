@@ -11,7 +11,9 @@ class EmuOps:
     def embedding(self, ids, table, scale=1.0):
         return table[ids.long()].float() * scale
 
-    def add_rms_norm(self, resid, delta, weight, eps, out_dtype, rows=None, delta2=None, groups=1):
+    def add_rms_norm(self, resid, delta, weight, eps, out_dtype, rows=None, delta2=None, groups=1, gate=None):
+        if gate is not None:
+            delta = delta.float() * gate[2] * torch.sigmoid(gate[0].float() + gate[1].float())
         if delta is not None and delta2 is not None:
             delta = delta.float() + delta2.float()
         if rows is None:

@@ -81,6 +81,13 @@ MER_REC = dict(architecture="Meronex", vocab=53, width=24, norm=dict(eps=1e-5, g
                layers=[_layer("mlstm", _mlstm(2, 4, 6, 9.0), _moe(8, 2.0, 4, 2)),
                        _layer("delta", _delta(2, 1, 4, 6, 3), _moe(8, 1.0, 3, 1))])
 
+#: sizes that are multiples of nothing: rows of the products that no vector load fits, heads of odd sizes
+MER_ODD = dict(architecture="Meronex", vocab=77, width=50, norm=dict(eps=1e-6, groups=5), residual_mult=0.45,
+               layers=[_layer("parallel", _parallel(_left(6, 3, 10, 7, 0.3, softcap=6.0, base=3000.0, dims=6,
+                                                          scaling=dict(factor=16.0, original=32, fast=3.0, slow=0.5)), 5, 7, 3), _moe(18, 1.2, 7, 3)),
+                       _layer("mlstm", _mlstm(5, 7, 9, 8.0), _moe(11, 2.0, 3, 2)),
+                       _layer("delta", _delta(6, 2, 5, 11, 5), _moe(13, 0.7, 9, 1))])
+
 INIT = dict(matrix_std=0.12, norm_std=0.2, bias_std=0.3)
 
 

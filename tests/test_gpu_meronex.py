@@ -62,7 +62,20 @@ def test_norm_in_groups_and_result_gate(dtype, T, H, groups):
     assert torch.equal(r2.cpu(), resid.float())
     y, pre, b = rnd(g, T, H).to(DT[dtype]), rnd(g, T, H + 7).to(DT[dtype]), rnd(g, H).to(DT[dtype])
     got = ops.sigmoid_gate(y.to(dev), pre.to(dev)[:, 3:3 + H], b.to(dev), 0.45)
-    close(got, y.double() * 0.45 * torch.sigmoid(pre.double()[:, 3:3 + H] + b.double()), DT[dtype], what="gate with bias and constant")
+    gated = y.double() * 0.45 * torch.sigmoid(pre.double()[:, 3:3 + H] + b.double())
+    close(got, gated, DT[dtype], what="gate with bias and constant")
+    # the same gate inside the kernel that sums the result into the stream and norms the sum, for all rows and for chosen ones
+    gate_rows = pre[:, 3:3 + H].contiguous()
+    wb = b.to(w.dtype)
+    x2 = resid.float().double() + y.double() * 0.45 * torch.sigmoid(gate_rows.double() + wb.double())
+    r3 = resid.float().to(dev)
+    out3 = ops.add_rms_norm(r3, y.to(dev), w.to(dev), 1e-5, DT[dtype], groups=groups, gate=(gate_rows.to(dev), wb.to(dev), 0.45))
+    close(r3, x2, torch.float32, what="stream after the gated addend")
+    close(out3, plain.grouped_norm(x2, w.double(), 1e-5, groups), DT[dtype], what="norm after the gated addend")
+    r4 = resid.float().to(dev)
+    out4 = ops.add_rms_norm(r4, y.to(dev), w.to(dev), 1e-5, DT[dtype], rows, groups=groups, gate=(gate_rows.to(dev), wb.to(dev), 0.45))
+    close(out4, plain.grouped_norm(x2, w.double(), 1e-5, groups)[[T - 1, 0]], DT[dtype], what="norm of chosen rows after the gated addend")
+    assert torch.equal(r4.cpu(), resid.float())
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -288,7 +301,7 @@ def test_experts_with_weighted_inputs_and_clamps(dtype, T, K, F, E, top):
 
 
 # ---- whole models ------------------------------------------------------------------------------
-MODELS = {"a": (mc.MER_A, 3, None), "b": (mc.MER_B, 4, None), "c": (mc.MER_C, 6, mc.decisive_router()), "a_sharp": (mc.MER_A, 5, mc.sharpen()),
+MODELS = {"odd": (mc.MER_ODD, 2, None), "a": (mc.MER_A, 3, None), "b": (mc.MER_B, 4, None), "c": (mc.MER_C, 6, mc.decisive_router()), "a_sharp": (mc.MER_A, 5, mc.sharpen()),
           "a_memory": (mc.MER_A, 9, mc.long_memory()), "c_memory": (mc.MER_C, 11, mc.both(mc.long_memory(w0=-3.0), mc.decisive_router())),
           "far_sharp": (mc.MER_FAR, 8, mc.both(mc.sharpen(8.0), mc.long_memory())), "c_sharp": (mc.MER_C, 12, mc.both(mc.sharpen(3.0), mc.long_memory()))}
 
@@ -299,7 +312,7 @@ def folders(tmp_path_factory):
 
 
 # (sharpened scores carry several times the rounding of a bfloat16 key: those models are held in float32 only)
-@pytest.mark.parametrize("name,dtype", [(n, d) for n in ("a", "b", "c", "a_sharp", "a_memory", "c_memory") for d in ("float32", "bfloat16")
+@pytest.mark.parametrize("name,dtype", [(n, d) for n in ("a", "b", "c", "odd", "a_sharp", "a_memory", "c_memory") for d in ("float32", "bfloat16")
                                         if not (n.endswith("sharp") and d == "bfloat16")])
 @pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
 def test_schedules_equal_the_plain_implementation(folders, name, mode, dtype, tmp_path):

@@ -18,7 +18,7 @@ TOL = dict(atol=3e-4, rtol=3e-4)
 def folders(tmp_path_factory):
     return {name: mc.write_model(str(tmp_path_factory.mktemp("mer_" + name)), cfg, seed, tweak, torch.float32)
             for name, cfg, seed, tweak in (("a", mc.MER_A, 3, None), ("b", mc.MER_B, 4, None), ("a_sharp", mc.MER_A, 5, mc.sharpen()),
-                                        ("a_memory", mc.MER_A, 9, mc.long_memory()))}
+                                        ("a_memory", mc.MER_A, 9, mc.long_memory()), ("odd", mc.MER_ODD, 2, None))}
 
 
 def test_configuration_is_read_by_name_and_checked():
@@ -81,7 +81,7 @@ def test_an_inner_size_that_no_key_names_comes_from_the_tensors(folders, emu_ops
     rc.compare(rc.collect(str(tmp_path / "out"), steps, 97), mc.plain_logits(folders["a"], requests), what="rank from tensors", **TOL)
 
 
-@pytest.mark.parametrize("name", ["a", "b", "a_sharp", "a_memory"])
+@pytest.mark.parametrize("name", ["a", "b", "a_sharp", "a_memory", "odd"])
 @pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
 def test_schedules_equal_the_plain_implementation(folders, name, mode, tmp_path, emu_ops):
     folder = folders[name]
