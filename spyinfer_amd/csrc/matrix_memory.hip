@@ -470,8 +470,10 @@ extern "C" int spy_causal_conv_silu(void* y, const void* x, long long xs, int dt
 template <typename TA, typename TW>
 __global__ __launch_bounds__(64) void delta_prepare_kernel(float* __restrict__ qk, const TA* __restrict__ qkv, float* __restrict__ beta,
                                                           float* __restrict__ dec, const TW* __restrict__ a_log,
-                                                          const TW* __restrict__ dt_bias, int H, int G, int d, int dv, int dd) {
-    // dd: decays per head, d (one per key channel) or 1 (one for the head)
+                                                          const TW* __restrict__ dt_bias, int H, int G, int d, int dv, int dd,
+                                                          long long bs, long long zs) {
+    // dd: decays per head, d (one per key channel) or 1 (one for the head); bs, zs: values from one token's row of beta
+    // and of the decays to the next (both may be columns of one wider product)
     const int t = blockIdx.x, unit = blockIdx.y, lane = threadIdx.x;
     const int C = 2 * G * d + H * dv;
     if (unit < G) {
@@ -496,16 +498,16 @@ __global__ __launch_bounds__(64) void delta_prepare_kernel(float* __restrict__ q
     }
     const int h = unit - G;
     const float rate = expf(to_f32<TW>(a_log[h]));
-    float* z = dec + ((size_t)t * H + h) * dd;
+    float* z = dec + (size_t)t * zs + (size_t)h * dd;
     for (int i = lane; i < dd; i += 64) z[i] = expf(-rate * softplus_f(z[i] + to_f32<TW>(dt_bias[(size_t)h * dd + i])));
-    if (lane == 0) beta[(size_t)t * H + h] = mm_sigmoid(beta[(size_t)t * H + h]);
+    if (lane == 0) beta[(size_t)t * bs + h] = mm_sigmoid(beta[(size_t)t * bs + h]);
 }
 
 template <typename TA, typename TW, int DR>
 __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
     float* __restrict__ o_out, float* __restrict__ state, long long state_stride, const TA* __restrict__ qkv, const float* __restrict__ qk,
     const float* __restrict__ beta_pre, const float* __restrict__ dec_pre, const int* __restrict__ cu_q,
-    const int* __restrict__ slot_ids, int num_slots, int H, int G, int d, int dv, int dd) {
+    const int* __restrict__ slot_ids, int num_slots, int H, int G, int d, int dv, int dd, long long bs, long long zs) {
     constexpr int R = (DR + MM_SLICE - 1) / MM_SLICE, LD = R * MM_SLICE, DQ = DR / 4;
     __shared__ __align__(16) float ks[LD], qs[LD], dec[LD];
     const int s = blockIdx.x, h = blockIdx.y, c = blockIdx.z, lane = threadIdx.x;
@@ -536,10 +538,10 @@ __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
             const int idx = lane + MM_SLICE * i;                                                 \
             qr[U][i] = idx < d ? qk_[(size_t)g * d + idx] : 0.f;                                 \
             kr[U][i] = idx < d ? qk_[(size_t)(G + g) * d + idx] : 0.f;                           \
-            zr[U][i] = idx < d ? dec_pre[((size_t)(TT) * H + h) * dd + (dd == 1 ? 0 : idx)] : 1.f; \
+            zr[U][i] = idx < d ? dec_pre[(size_t)(TT) * zs + (size_t)h * dd + (dd == 1 ? 0 : idx)] : 1.f; \
         }                                                                                        \
         vr[U] = col ? to_f32<TA>(qkv[(size_t)(TT) * C + (size_t)2 * G * d + (size_t)h * dv + j]) : 0.f; \
-        br[U] = beta_pre[(size_t)(TT) * H + h];                                                  \
+        br[U] = beta_pre[(size_t)(TT) * bs + h];                                                 \
     }
 #pragma unroll
     for (int u = 0; u < MM_AHEAD; ++u) DELTA_LOAD(u, t0 + u)
@@ -590,19 +592,20 @@ __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
 extern "C" int spy_delta_rule(void* out, float* o_tmp, float* qk_tmp, float* state, long long state_stride, const void* qkv, int dtype,
                               float* beta_pre, float* dec_pre, const void* a_log, const void* dt_bias, int w_dtype, const void* gate, long long gs,
                               const void* norm_w, float eps, const int* cu_q, const int* slot_ids, int num_slots, int S, int T, int H,
-                              int G, int d, int dv, int dd, int silu_gate, hipStream_t st) {
+                              int G, int d, int dv, int dd, int silu_gate, long long bs, long long zs, hipStream_t st) {
     SPY_REQUIRE(S > 0 && T > 0 && H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0 && num_slots > 0 && o_tmp, "spy_delta_rule: empty operand");
     SPY_REQUIRE(dd == d || dd == 1, "spy_delta_rule: %d decays for a head of %d key channels (one, or one per channel)", dd, d);
+    SPY_REQUIRE(bs >= H && zs >= (long long)H * dd, "spy_delta_rule: rows of beta or of the decays are too short");
     SPY_REQUIRE(d <= 256 && dv <= 1024 && H <= 65535, "spy_delta_rule: heads of %d x %d (key size up to 256, value size up to 1024)", d, dv);
     SPY_REQUIRE(state_stride >= (long long)H * d * dv && gs >= (long long)H * dv, "spy_delta_rule: the state or the gate rows are too short");
     SPY_REQUIRE(qk_tmp && G + H <= 65535, "spy_delta_rule: no room for the unit vectors");
     const dim3 pgrid(T, G + H);
     SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (delta_prepare_kernel<TA, TW><<<pgrid, 64, 0, st>>>(
-        qk_tmp, (const TA*)qkv, beta_pre, dec_pre, (const TW*)a_log, (const TW*)dt_bias, H, G, d, dv, dd))));
+        qk_tmp, (const TA*)qkv, beta_pre, dec_pre, (const TW*)a_log, (const TW*)dt_bias, H, G, d, dv, dd, bs, zs))));
     SPY_CHECK_LAUNCH("spy_delta_rule (unit vectors and decays)");
     const dim3 grid(S, H, (dv + MM_COLS - 1) / MM_COLS);
     SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, MM_LAUNCH(delta_rule_kernel, o_tmp, state, state_stride, (const TA*)qkv, qk_tmp, beta_pre,
-        dec_pre, cu_q, slot_ids, num_slots, H, G, d, dv, dd)));
+        dec_pre, cu_q, slot_ids, num_slots, H, G, d, dv, dd, bs, zs)));
     SPY_CHECK_LAUNCH("spy_delta_rule");
     const dim3 ngrid(T, H);
     const int nthreads = dv >= 256 ? 256 : 64;
@@ -661,14 +664,17 @@ extern "C" int spy_token_shift(void* out, const void* x, int dtype, const void* 
     return 0;
 }
 
-__global__ void tanh_kernel(float* __restrict__ x, long long n) {
-    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) x[i] = tanhf(x[i]);
+template <typename TC>
+__global__ void tanh_kernel(TC* __restrict__ out, const float* __restrict__ x, long long n) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
+        out[i] = from_f32<TC>(tanhf(x[i]));
 }
 
-extern "C" int spy_tanh(float* x, long long n, hipStream_t st) {
+// out = tanh(x) of float32 sums, rounded once to the dtype that the next product reads
+extern "C" int spy_tanh(void* out, int dtype, const float* x, long long n, hipStream_t st) {
     SPY_REQUIRE(n > 0, "spy_tanh: empty operand");
     const unsigned blocks = (unsigned)((n + 255) / 256 > 65536 ? 65536 : (n + 255) / 256);
-    tanh_kernel<<<blocks, 256, 0, st>>>(x, n);
+    SPY_DISPATCH(dtype, TC, (tanh_kernel<TC><<<blocks, 256, 0, st>>>((TC*)out, x, n)));
     SPY_CHECK_LAUNCH("spy_tanh");
     return 0;
 }

@@ -1317,8 +1317,9 @@ def delta_rule(qkv: torch.Tensor, beta_pre: torch.Tensor, dec_pre: torch.Tensor,
     [T, H dv]: o over its root mean square, times ``norm_w [dv]``, times sigmoid(``gate``) (rows of H dv values, a view
     into a wider product allowed; ``gate_act`` "silu": times silu(gate)).  One decay per head instead of one per key
     channel: ``dec_pre [T, H]`` and ``dt_bias [H]``."""
-    _dev(qkv, beta_pre, dec_pre, a_log, dt_bias, norm_w, state, cu_q, slot_ids)
+    _dev(qkv, a_log, dt_bias, norm_w, state, cu_q, slot_ids)
     gs = _row_view(gate, "delta_rule")
+    bs, zs = _row_view(beta_pre, "delta_rule"), _row_view(dec_pre, "delta_rule")       # (both may be columns of one wider product)
     T = qkv.shape[0]
     S = _entries(cu_q, slot_ids, "delta_rule")
     _check(qkv.dim() == 2 and qkv.shape[1] == 2 * G * d + H * dv and qkv.dtype in _CODES and gate.dtype == qkv.dtype and gate.shape == (T, H * dv),
@@ -1336,11 +1337,11 @@ def delta_rule(qkv: torch.Tensor, beta_pre: torch.Tensor, dec_pre: torch.Tensor,
     if T:
         tmp = torch.empty((T, H * dv), dtype=torch.float32, device=qkv.device)      # the read-outs before the heads' norm
         unit = torch.empty((T, 2 * G * d), dtype=torch.float32, device=qkv.device)  # q and k as unit vectors
-        hip().call("spy_delta_rule", _ptr(out), _ptr(tmp), _ptr(unit), _ptr(state), ctypes.c_longlong(state.shape[1]), _ptr(qkv), _code(qkv, "qkv"), _ptr(beta_pre),
-                   _ptr(dec_pre), _ptr(a_log), _ptr(dt_bias), _code(a_log, "decay numbers"), ctypes.c_void_p(gate.data_ptr()), ctypes.c_longlong(gs),
+        hip().call("spy_delta_rule", _ptr(out), _ptr(tmp), _ptr(unit), _ptr(state), ctypes.c_longlong(state.shape[1]), _ptr(qkv), _code(qkv, "qkv"),
+                   ctypes.c_void_p(beta_pre.data_ptr()), ctypes.c_void_p(dec_pre.data_ptr()), _ptr(a_log), _ptr(dt_bias), _code(a_log, "decay numbers"), ctypes.c_void_p(gate.data_ptr()), ctypes.c_longlong(gs),
                    _ptr(norm_w), ctypes.c_float(eps), _ptr(cu_q), _ptr(slot_ids), ctypes.c_int(state.shape[0]), ctypes.c_int(S), ctypes.c_int(T),
                    ctypes.c_int(H), ctypes.c_int(G), ctypes.c_int(d), ctypes.c_int(dv), ctypes.c_int(dd), ctypes.c_int(1 if gate_act == "silu" else 0),
-                   _Hip.stream())
+                   ctypes.c_longlong(bs), ctypes.c_longlong(zs), _Hip.stream())
     return out
 
 
@@ -1364,13 +1365,14 @@ def token_shift(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, keep_off
     return out
 
 
-def tanh_(x: torch.Tensor) -> torch.Tensor:
-    """tanh in place over a float32 tensor."""
+def tanh_cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """tanh of a float32 tensor, rounded once to ``dtype`` (what the next product reads)."""
     _dev(x)
-    _check(x.dtype == torch.float32, "tanh_: float32 expected")
+    _check(x.dtype == torch.float32 and dtype in _CODES, "tanh_cast: float32 in, float32 or bfloat16 out")
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
     if x.numel():
-        hip().call("spy_tanh", _ptr(x), ctypes.c_longlong(x.numel()), _Hip.stream())
-    return x
+        hip().call("spy_tanh", _ptr(out), _code(out, "out"), _ptr(x), ctypes.c_longlong(x.numel()), _Hip.stream())
+    return out
 
 
 def time_mix(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, dec_pre: torch.Tensor, w0: torch.Tensor, u: torch.Tensor, gate: torch.Tensor,

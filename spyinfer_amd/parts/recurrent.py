@@ -310,7 +310,7 @@ class HeadDelta(Mixer):
         H, G, d, dv, C = self.heads, self.kv_heads, self.dim, self.vdim, self._channels()
         proj = ops.linear_few(x, self.w_in, self.w_in_tiled)
         small = ops.linear(x, self.w_small, torch.float32)                    # [beta | decay], float32 sums kept
-        beta_pre, dec_pre = small[:, :H].contiguous(), small[:, H:].contiguous()
+        beta_pre, dec_pre = small[:, :H], small[:, H:]                        # (the walk's kernels read them where they lie)
         cu_q, slots = batch.array("cu_q"), batch.array("slot_ids")
         qkv = ops.causal_conv_silu(proj[:, :C], self.taps, cache.state, H * d * dv, batch.array("token_entry"), cu_q, slots)
         y = ops.delta_rule(qkv, beta_pre, dec_pre, self.a_log, self.dt_bias, proj[:, C:], self.norm, self.norm_eps, cache.state, cu_q, slots,
@@ -369,8 +369,8 @@ class TimeMix(Mixer):
         cu_q, slots = batch.array("cu_q"), batch.array("slot_ids")
         blends = ops.token_shift(x, self.mu, cache.state, H * d * d, batch.array("token_entry"), cu_q, slots)      # [5, T, W]
         r, k, v, g = (ops.linear_few(blends[i], w[0], w[1]) for i, w in enumerate((self.w_r, self.w_k, self.w_v, self.w_g)))
-        inner = ops.tanh_(ops.linear(blends[4], self.w_1, torch.float32))
-        # (the inner projection's result is an activation: it takes the activation dtype on its way into the outer one)
-        dec_pre = ops.linear(inner.to(self.w_2.dtype).contiguous(), self.w_2, torch.float32)
+        # (the inner projection's result is an activation: it takes the outer matrix's dtype on its way into that product)
+        inner = ops.tanh_cast(ops.linear(blends[4], self.w_1, torch.float32), self.w_2.dtype)
+        dec_pre = ops.linear(inner, self.w_2, torch.float32)
         y = ops.time_mix(r, k, v, dec_pre, self.w0, self.u, g, self.norm, self.norm_eps, cache.state, cu_q, slots, H, d)
         return ops.linear_few(y, self.w_o[0], self.w_o[1])

@@ -23,7 +23,7 @@ def emu_ops(monkeypatch):
     emu = EmuOps()
     for name in ("embedding", "add_rms_norm", "rms_norm", "qk_norm_rope_store", "swiglu", "sample", "pair_embedding", "norm_residual",
                  "depth_mix", "xielu", "mingru", "gemm_strided", "latent_prepare", "latent_attention", "bias_rope_store", "sigmoid_gate",
-                 "mlstm", "causal_conv_silu", "delta_rule", "moe_route", "moe_experts", "token_shift", "tanh_", "time_mix", "norm_pair_mean"):
+                 "mlstm", "causal_conv_silu", "delta_rule", "moe_route", "moe_experts", "token_shift", "tanh_cast", "time_mix", "norm_pair_mean"):
         monkeypatch.setattr(ops, name, getattr(emu, name))
 
     def linear(x, w, out_dtype=None, tiled=None, out=None):

@@ -337,8 +337,8 @@ class EmuOps:
             keep.copy_(f[t1 - 1])
         return (f[None] + (prev - f)[None] * mu.float()[:, None, :]).to(x.dtype)
 
-    def tanh_(self, x):
-        return x.copy_(torch.tanh(x))
+    def tanh_cast(self, x, dtype):
+        return torch.tanh(x).to(dtype)
 
     def time_mix(self, r, k, v, dec_pre, w0, u, gate, norm_w, eps, state, cu_q, slot_ids, H, d):
         T = r.shape[0]
