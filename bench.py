@@ -102,10 +102,10 @@ def meronex_shape(width: int, layers: int, vocab: int) -> dict:
     of 128, values of 256, half as many heads), a delta rule with one decay per head (heads of 128 x 128, half as many q/k
     heads, 4 taps) and an attention (heads of 128 with 64 rotated dims, a quarter as many kv heads, capped scores) beside
     a time mix (heads of 64, a decay of inner size 64); every feed-forward 32 experts of 3/4 width of which a token uses
-    four (as many active weights as a dense layer of three times the width); norms in 4 groups."""
+    four (as many active weights as a dense layer of three times the width); norms in 8 groups."""
     heads = max(1, width // 128)
     rot = dict(base=500000.0, dims=64, scaling=dict(factor=8.0, original=8192, fast=32.0, slow=1.0))
-    left = dict(heads=heads, kv_heads=max(1, heads // 4), dim=128, vdim=128, scale=128 ** -0.5, softcap=50.0, rot=rot)
+    left = dict(heads=heads, kv_heads=max(1, heads // 4), dim=128, vdim=128, scale=128 ** -0.5, softcap=30.0, rot=rot)
     moe = dict(kind="moe", expert=dict(ff=3 * width // 4, limit=7.0), router=dict(experts=32, top=4))
     out = []
     for i in range(layers):
@@ -116,12 +116,14 @@ def meronex_shape(width: int, layers: int, vocab: int) -> dict:
             out.append(dict(type="delta", mixer=dict(heads=heads, kv_heads=max(1, heads // 2), dim=128, vdim=128, conv=4), mlp=moe))
         else:
             out.append(dict(type="parallel", mixer=dict(left=dict(left), right=dict(heads=max(1, width // 64), dim=64, decay_rank=64)), mlp=moe))
-    return dict(architecture="Meronex", vocab=vocab, width=width, norm=dict(eps=1e-6, groups=4), residual_mult=0.5, layers=out)
+    return dict(architecture="Meronex", vocab=vocab, width=width, norm=dict(eps=1e-5, groups=8), residual_mult=0.7, layers=out)
 
 
 DESIGN_SHAPES = {"sefevik": ("Sefevik", sefevik_shape), "sodedra": ("Sodedra", sodedra_shape), "meronex": ("Meronex", meronex_shape)}
 #: further designs that a design is measured beside (Qwen3 always is): the closest one the engine has
 DESIGN_BESIDE = {"meronex": ("sodedra",)}
+#: layers, where --layers does not say: a whole number of the design's turns of layer kinds
+DESIGN_LAYERS = {"meronex": 9}
 
 
 def design_compare(args) -> int:
@@ -140,7 +142,7 @@ def design_compare(args) -> int:
 
     ops.hip()
     dev = torch.device("cuda:0")
-    layers, vocab, page = args.layers or 8, 32768, 16
+    layers, vocab, page = args.layers or DESIGN_LAYERS.get(design, 8), 32768, 16
     run_dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
     g = torch.Generator().manual_seed(args.seed)
     results = {}

@@ -107,26 +107,6 @@ extern "C" int spy_embedding_sumsq(float* out, void* xw, float* ss, const void* 
 // One block per row.  The row is read once and kept in registers (4 values per thread and pass,
 // up to NORM_PASSES passes); longer rows are read again for the second pass.
 #define NORM_PASSES 8
-template <typename TA> struct Vec4;
-template <> struct Vec4<float> {
-    typedef float4 type;
-    static __device__ __forceinline__ void load(const float* p, float* v) { const float4 t = *reinterpret_cast<const float4*>(p); v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
-    static __device__ __forceinline__ void store(float* p, const float* v) { *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]); }
-};
-template <> struct Vec4<bf16_t> {
-    static __device__ __forceinline__ void load(const bf16_t* p, float* v) {
-        const uint2 t = *reinterpret_cast<const uint2*>(p);
-        v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
-        v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
-    }
-    static __device__ __forceinline__ void store(bf16_t* p, const float* v) {
-        uint2 t;
-        t.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
-        t.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
-        *reinterpret_cast<uint2*>(p) = t;
-    }
-};
-
 template <typename TA, typename TW, bool VEC>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restrict__ delta, const TA* __restrict__ delta2,
                                    const TW* __restrict__ w, float eps, TA* __restrict__ out, const int* __restrict__ rows, int T,

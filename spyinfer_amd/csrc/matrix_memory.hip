@@ -800,23 +800,57 @@ extern "C" int spy_time_mix(void* out, float* o_tmp, float* bonus, float* state,
 }
 
 // ---- two results normed over the width and averaged ----------------------------------------------------------------------
-// out[t] = (a[t] / rms(a[t]) * wa + b[t] / rms(b[t]) * wb) / 2; one block per row
-template <typename TA, typename TW>
+// out[t] = (a[t] / rms(a[t]) * wa + b[t] / rms(b[t]) * wb) / 2; one block per row.  VEC: W % 4 == 0, aligned rows, and a row
+// fits PAIR_PASSES passes of four values a thread: both rows are read once and stay in registers
+#define PAIR_PASSES 4
+template <typename TA, typename TW, bool VEC>
 __global__ void norm_pair_mean_kernel(TA* __restrict__ out, const TA* __restrict__ a, const TA* __restrict__ b, const TW* __restrict__ wa,
                                       const TW* __restrict__ wb, float eps, int W) {
-    __shared__ float red[16];
+    __shared__ float red[16], red2[16];
     const TA* ar = a + (size_t)blockIdx.x * W;
     const TA* br = b + (size_t)blockIdx.x * W;
+    TA* o = out + (size_t)blockIdx.x * W;
     float sa = 0.f, sb = 0.f;
+    if (VEC) {
+        float x[PAIR_PASSES][4], y[PAIR_PASSES][4];
+#pragma unroll
+        for (int p = 0; p < PAIR_PASSES; ++p) {
+            const int i = (p * blockDim.x + threadIdx.x) * 4;
+            if (i < W) {
+                Vec4<TA>::load(ar + i, x[p]);
+                Vec4<TA>::load(br + i, y[p]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    sa = fmaf(x[p][e], x[p][e], sa);
+                    sb = fmaf(y[p][e], y[p][e], sb);
+                }
+            }
+        }
+        sa = block_sum(sa, red);
+        sb = block_sum(sb, red2);
+        const float ra = 0.5f / sqrtf(sa / (float)W + eps), rb = 0.5f / sqrtf(sb / (float)W + eps);
+#pragma unroll
+        for (int p = 0; p < PAIR_PASSES; ++p) {
+            const int i = (p * blockDim.x + threadIdx.x) * 4;
+            if (i < W) {
+                float u4[4], v4[4], r4[4];
+                Vec4<TW>::load(wa + i, u4);
+                Vec4<TW>::load(wb + i, v4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) r4[e] = fmaf(x[p][e] * ra, u4[e], (y[p][e] * rb) * v4[e]);
+                Vec4<TA>::store(o + i, r4);
+            }
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < W; i += blockDim.x) {
         const float x = to_f32<TA>(ar[i]), y = to_f32<TA>(br[i]);
         sa = fmaf(x, x, sa);
         sb = fmaf(y, y, sb);
     }
     sa = block_sum(sa, red);
-    sb = block_sum(sb, red);
+    sb = block_sum(sb, red2);
     const float ra = 0.5f / sqrtf(sa / (float)W + eps), rb = 0.5f / sqrtf(sb / (float)W + eps);
-    TA* o = out + (size_t)blockIdx.x * W;
     for (int i = threadIdx.x; i < W; i += blockDim.x)
         o[i] = from_f32<TA>(fmaf(to_f32<TA>(ar[i]) * ra, to_f32<TW>(wa[i]), (to_f32<TA>(br[i]) * rb) * to_f32<TW>(wb[i])));
 }
@@ -824,9 +858,16 @@ __global__ void norm_pair_mean_kernel(TA* __restrict__ out, const TA* __restrict
 extern "C" int spy_norm_pair_mean(void* out, const void* a, const void* b, int dtype, const void* wa, const void* wb, int w_dtype, float eps,
                                   int T, int W, hipStream_t st) {
     SPY_REQUIRE(T > 0 && W > 0, "spy_norm_pair_mean: empty operand");
-    const int threads = W >= 1024 ? 256 : 64;
-    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (norm_pair_mean_kernel<TA, TW><<<T, threads, 0, st>>>(
-        (TA*)out, (const TA*)a, (const TA*)b, (const TW*)wa, (const TW*)wb, eps, W))));
+    const int threads = W >= 2048 ? 256 : (W >= 512 ? 128 : 64);
+    const bool vec = W % 4 == 0 && W <= threads * 4 * PAIR_PASSES && ((uintptr_t)out % 16) == 0 && ((uintptr_t)a % 16) == 0 &&
+                     ((uintptr_t)b % 16) == 0 && ((uintptr_t)wa % 16) == 0 && ((uintptr_t)wb % 16) == 0;
+    if (vec) {
+        SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (norm_pair_mean_kernel<TA, TW, true><<<T, threads, 0, st>>>(
+            (TA*)out, (const TA*)a, (const TA*)b, (const TW*)wa, (const TW*)wb, eps, W))));
+    } else {
+        SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (norm_pair_mean_kernel<TA, TW, false><<<T, 256, 0, st>>>(
+            (TA*)out, (const TA*)a, (const TA*)b, (const TW*)wa, (const TW*)wb, eps, W))));
+    }
     SPY_CHECK_LAUNCH("spy_norm_pair_mean");
     return 0;
 }
