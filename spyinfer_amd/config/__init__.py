@@ -1,4 +1,4 @@
 from .engine_config import EngineConfig
-from .model_config import ConfigError, ModelConfig, MeronexConfig, Qwen3Config, SefevikConfig, SodedraConfig
+from .model_config import ConfigError, ModelConfig, MeronexConfig, Qwen3Config, SefevikConfig, SodedraConfig, TarunexConfig
 from .registry import (Architecture, architecture_of, get_architecture, load_model_config,
                        register_architecture, registered_architectures, unregister_architecture)

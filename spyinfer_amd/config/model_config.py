@@ -527,3 +527,121 @@ class MeronexConfig(ModelConfig):
             f = layer["mlp"]
             if f and (f["ff"] <= 0 or not f["limit"] > 0.0 or f["experts"] <= 0 or not 0 < f["top"] <= f["experts"]):
                 raise ConfigError("%s.mlp: inner size and limit positive, 1 to %d choices" % (where, max(f["experts"], 1)))
+
+
+@dataclasses.dataclass
+class TarunexConfig(ModelConfig):
+    """Tarunex: layers whose mixer and feed-forward read the stream through a norm each (a norm's weight is one number)
+    and are added together; a run of consecutive layers may be walked several times with the same weights (``loop``),
+    every walk with caches of its own, the embedding output added back before every walk but the first and a learned
+    vector before each; token mixers 'attention' (grouped queries with biases and no rotation, a temperature on the
+    queries that grows with the logarithm of the position, capped scores lowered by a logarithmic penalty on the
+    distance, a softmax with a one in its denominator, one gate number per head) and 'latent_attention' (queries through
+    a normed low-rank vector, keys and values expanded from a cached one, interleaved rotary pairs on a part that all
+    heads share, one gate number per head); the feed-forward a mixture of gated experts (a router with a bias, the
+    weights a softmax over the chosen logits) plus an expert that every token uses; scaled and capped logits.  The
+    configuration is nested; ``layers`` lists every layer's type and sizes, and nothing is assumed equal between layers."""
+
+    architecture: str = ""
+    vocab: int = -1
+    width: int = -1
+    norm_eps: float = 0.0
+    embedding_scale: float = 1.0
+    logit_scale: float = 1.0
+    logit_softcap: float = 0.0
+    #: None, or {start, stop, times}: layers start .. stop - 1 are walked ``times`` times in a row
+    loop: Optional[Dict[str, int]] = None
+    #: one dict per layer: type, mixer (sizes and constants of that mixer), mlp (None or {kind: moe, ff, experts, top, shared_ff})
+    layers: List[Dict[str, Any]] = dataclasses.field(default_factory=list)
+
+    MIXERS: ClassVar[tuple] = ("attention", "latent_attention")
+
+    @classmethod
+    def from_dict(cls, raw: Dict[str, Any]) -> "TarunexConfig":
+        cfg = cls(architecture=str(raw.get("architecture") or (raw.get("architectures") or [""])[0]),
+                  vocab=_need(raw, "vocab", int), width=_need(raw, "width", int), norm_eps=float(_need(raw, "norm.eps", (int, float))))
+        if (raw.get("embedding") or {}).get("scale") is not None:
+            cfg.embedding_scale = float(_need(raw, "embedding.scale", (int, float)))
+        if raw.get("logit_scale") is not None:
+            cfg.logit_scale = float(_need(raw, "logit_scale", (int, float)))
+        if raw.get("logit_softcap") is not None:
+            cfg.logit_softcap = float(_need(raw, "logit_softcap", (int, float)))
+        if raw.get("loop"):
+            cfg.loop = {k: _need(raw, "loop." + k, int) for k in ("start", "stop", "times")}
+        cfg.layers = [cls._layer(i, l) for i, l in enumerate(_need(raw, "layers", list))]
+        cfg._raw = dict(raw)
+        cfg.validate()
+        return cfg
+
+    @classmethod
+    def _layer(cls, i: int, raw: Dict[str, Any]) -> Dict[str, Any]:
+        where = "config.json layers[%d]" % i
+        if not isinstance(raw, dict):
+            raise ConfigError("%s is no object" % where)
+        kind = _need(raw, "type", str, where)
+        if kind not in cls.MIXERS:
+            raise ConfigError("%s: mixer type %r is not known (%s)" % (where, kind, ", ".join(cls.MIXERS)))
+        m = _need(raw, "mixer", dict, where)
+        at = where + ".mixer"
+        if kind == "attention":
+            mix = {k: _need(m, k, int, at) for k in ("heads", "dim", "vdim")}
+            mix["kv_heads"] = _need(m, "kv_heads", int, at) if m.get("kv_heads") is not None else mix["heads"]
+            mix["scale"] = float(_need(m, "scale", (int, float), at))
+            mix["softcap"] = float(_need(m, "softcap", (int, float), at)) if m.get("softcap") is not None else 0.0
+            mix["q_temp"] = None
+            if m.get("q_temp"):
+                mix["q_temp"] = {"coef": float(_need(m, "q_temp.coef", (int, float), at)), "every": _need(m, "q_temp.every", int, at)}
+        else:
+            mix = {k: _need(m, k, int, at) for k in ("heads", "dim", "rot_dim", "vdim", "kv_rank", "q_rank")}
+            mix["scale"] = float(_need(m, "scale", (int, float), at))
+            rot = m.get("rot")
+            mix["rot"] = None
+            if rot:
+                mix["rot"] = {"base": float(_need(rot, "base", (int, float), at + ".rot")), "dims": _need(rot, "dims", int, at + ".rot")}
+        out = {"type": kind, "mixer": mix, "mlp": None}
+        mlp = raw.get("mlp")
+        if mlp is not None:
+            at = where + ".mlp"
+            fk = _need(mlp, "kind", str, at)
+            if fk != "moe":
+                raise ConfigError("%s: kind %r is not known (moe)" % (at, fk))
+            out["mlp"] = {"kind": fk, "ff": _need(mlp, "expert.ff", int, at), "experts": _need(mlp, "router.experts", int, at),
+                          "top": _need(mlp, "router.top", int, at),
+                          "shared_ff": _need(mlp, "shared.ff", int, at) if mlp.get("shared") else None}
+        return out
+
+    def to_dict(self) -> Dict[str, Any]:
+        return dict(getattr(self, "_raw", {}))
+
+    def validate(self) -> None:
+        if self.vocab <= 0 or self.width <= 0:
+            raise ConfigError("config.json: vocab and width must be positive")
+        if not (self.norm_eps > 0.0):
+            raise ConfigError("config.json: norm.eps must be positive")
+        if self.logit_softcap < 0.0:
+            raise ConfigError("config.json: logit_softcap must not be negative")
+        if not self.layers:
+            raise ConfigError("config.json: no layers")
+        if self.loop is not None:
+            lp = self.loop
+            if not (0 <= lp["start"] < lp["stop"] <= len(self.layers)) or lp["times"] < 1:
+                raise ConfigError("config.json loop: layers %d .. %d of %d, %d times" % (lp["start"], lp["stop"] - 1, len(self.layers), lp["times"]))
+        for i, layer in enumerate(self.layers):
+            where = "config.json layers[%d]" % i
+            m = layer["mixer"]
+            if any(isinstance(v, int) and not isinstance(v, bool) and v <= 0 for k, v in m.items() if k != "dim"):
+                raise ConfigError("%s.mixer: sizes must be positive" % where)
+            if layer["type"] == "attention":
+                if m["dim"] <= 0 or m["heads"] % m["kv_heads"]:
+                    raise ConfigError("%s.mixer: heads (%d) is not a multiple of kv_heads (%d)" % (where, m["heads"], m["kv_heads"]))
+                if m["softcap"] < 0.0:
+                    raise ConfigError("%s.mixer.softcap must not be negative" % where)
+                if m["q_temp"] and m["q_temp"]["every"] <= 0:
+                    raise ConfigError("%s.mixer.q_temp.every must be positive" % where)
+            else:
+                rot = m["rot"]
+                if m["dim"] < 0 or (rot and (rot["dims"] % 2 or not (0 < rot["dims"] <= m["rot_dim"]) or not rot["base"] > 1.0)):
+                    raise ConfigError("%s.mixer.rot: dims must be even and at most rot_dim, base above 1" % where)
+            f = layer["mlp"]
+            if f and (f["ff"] <= 0 or f["experts"] <= 0 or not 0 < f["top"] <= f["experts"] or (f["shared_ff"] is not None and f["shared_ff"] <= 0)):
+                raise ConfigError("%s.mlp: inner sizes positive, 1 to %d choices" % (where, max(f["experts"], 1)))

@@ -12,7 +12,10 @@ template <typename TA>
 __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
     TA* __restrict__ out, const TA* __restrict__ q, const TA* __restrict__ kc, const TA* __restrict__ vc, int P, int num_pages,
     const int* __restrict__ kv_len, const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_entry,
-    const int* __restrict__ positions, int n_q, int n_kv, int d, float scale, int window, float softcap) {
+    const int* __restrict__ positions, int n_q, int n_kv, int d, float scale, int window, float softcap,
+    const float* __restrict__ dist, int sink) {
+    // dist != null: [2, n_q] float32, a penalty on the distance taken off every (capped) score: dist[h] ln(1 + dist[n_q + h] (p - key)).
+    // sink: the softmax's denominator holds one more term, e^0, that has no value (a running maximum that starts at 0 with a sum of 1).
     __shared__ float qs[AG_MAX_D];
     __shared__ float ps[AG_THREADS];
     __shared__ int pg[AG_THREADS];
@@ -28,7 +31,8 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
     const TA* qv = q + ((size_t)t * n_q + h) * d;
     for (int j = tid; j < d; j += AG_THREADS) qs[j] = to_f32<TA>(qv[j]);
     float acc[AG_MAX_D / AG_THREADS] = {};
-    float m = -INFINITY, l = 0.f;
+    float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+    const float d1 = dist ? dist[h] : 0.f, d2 = dist ? dist[n_q + h] : 0.f;
     const int* bt = block_table + (size_t)s * max_blocks;
     __syncthreads();
     for (int c0 = lo; c0 <= hi; c0 += AG_THREADS) {
@@ -44,6 +48,7 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
                 for (int j = 0; j < d; ++j) dot = fmaf(qs[j], to_f32<TA>(kr[j]), dot);
                 sc = dot * scale;
                 if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
+                if (dist) sc -= d1 * log1pf(d2 * (float)(p - c));
             } else {
                 page = -1;   // a key without a page is not read (never the case for a checked batch)
             }
@@ -81,7 +86,7 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
 extern "C" int spy_attention_generic(void* out, const void* q, int dtype, const void* kc, const void* vc, int P, int num_pages,
                                      const int* kv_len, const int* block_table, int max_blocks, const int* token_entry,
                                      const int* positions, int S, int T, int n_q, int n_kv, int d, float scale, int window,
-                                     float softcap, hipStream_t st) {
+                                     float softcap, const float* dist, int sink, hipStream_t st) {
     SPY_REQUIRE(T > 0 && S > 0 && n_q > 0 && n_kv > 0 && d > 0 && P > 0 && num_pages > 0 && max_blocks > 0,
                 "spy_attention_generic: empty operand");
     SPY_REQUIRE(d <= AG_MAX_D, "spy_attention_generic: head_dim %d exceeds the supported %d", d, AG_MAX_D);
@@ -89,7 +94,7 @@ extern "C" int spy_attention_generic(void* out, const void* q, int dtype, const 
     const dim3 grid(T, n_q);
     SPY_DISPATCH(dtype, TA, (attention_generic_kernel<TA><<<grid, AG_THREADS, 0, st>>>(
         (TA*)out, (const TA*)q, (const TA*)kc, (const TA*)vc, P, num_pages, kv_len, block_table, max_blocks, token_entry,
-        positions, n_q, n_kv, d, scale, window, softcap)));
+        positions, n_q, n_kv, d, scale, window, softcap, dist, sink)));
     SPY_CHECK_LAUNCH("spy_attention_generic");
     return 0;
 }

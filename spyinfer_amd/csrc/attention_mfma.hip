@@ -133,7 +133,10 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
     int n_q, int n_kv, int d, float scale, int window, float softcap, int splits, float* __restrict__ ws, FusedQKV fz, int out_tiles,
-    unsigned* counters, int log2p, const int* __restrict__ pieces) {
+    unsigned* counters, int log2p, const int* __restrict__ pieces, const float* __restrict__ dist, int sink) {
+    // dist != null: [2, n_q] float32, a penalty on the distance taken off every (capped) score: dist[h] ln(1 + dist[n_q + h] (pos - key)).
+    // sink: the softmax's denominator holds one more term, e^0, that has no value: the first wave of the keys' first part
+    // starts its running maximum at 0 with a sum of 1 (in one of a row's four lanes, whose sums are added at the end).
     constexpr int KK = DMAX / 32;   // 32-wide chunks of the head dim for Q.K
     constexpr int DT = DMAX / 16;   // 16-row tiles of the head dim for P.V
     const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
@@ -202,6 +205,8 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
+    if (sink && sp == 0 && wave == 0 && row_ok) { m = 0.f; l = g == 0 ? 1.f : 0.f; }
+    const float d1 = dist ? dist[head] : 0.f, d2 = dist ? dist[n_q + head] : 0.f;
 
     // FUSED: the entry's one new token lies at position p0 = kvl - 1; its query rows have that position too.  The block
     // whose keys reach it prepares the new key (every lane its pieces for its g, as for q) and takes the new value's
@@ -396,6 +401,7 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
             const int key = c0 + 8 * g + j;
             float v = (j < 4 ? sa[j] : sb[j - 4]) * scale;
             if (softcap > 0.f) v = softcap * capped_tanh(v * inv_cap);          // scores capped: cap tanh(score / cap)
+            if (dist) v -= d1 * __logf(fmaf(d2, (float)max(pos - key, 0), 1.0f));
             const bool ok = row_ok && key <= pos && key >= lo_row && key < kvl;
             sc[j] = ok ? v : -INFINITY;
             bmax = fmaxf(bmax, sc[j]);
@@ -657,7 +663,9 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
                                   const int* tile_row0, int num_tiles, int S, int T, int n_q, int n_kv, int d, float scale,
                                   int window, float softcap, int splits, float* ws, const void* qkv, const void* qw, const void* kw, int w_dtype,
                                   float eps, const float* cos_t, const float* sin_t, int max_pos, int store, int out_tiles,
-                                  unsigned* counters, int n_counters, const int* pieces, int num_pieces, hipStream_t st) {
+                                  unsigned* counters, int n_counters, const int* pieces, int num_pieces, const float* dist, int sink,
+                                  hipStream_t st) {
+    SPY_REQUIRE(!qkv || (!dist && !sink), "spy_attention_mfma: the fused variant takes neither a penalty on the distance nor a sink");
     SPY_REQUIRE(num_tiles > 0 && S > 0 && T > 0 && n_q > 0 && n_kv > 0 && num_pages > 0 && max_blocks > 0,
                 "spy_attention_mfma: empty operand");
     SPY_REQUIRE(d % 16 == 0 && d >= 16 && d <= 256, "spy_attention_mfma: head_dim %d is not a multiple of 16 in 16..256", d);
@@ -698,7 +706,7 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
 #define ATT_LAUNCH(DM, FZ, FL)                                                                                                \
     attention_mfma_kernel<DM, FZ, FL><<<grid, AW * 64, (DM <= 128 ? AW : AW - 1) * ((DM / 16) * 4 + 2) * 64 * sizeof(float), st>>>(  \
         (bf16_t*)out, (const bf16_t*)q, (bf16_t*)kc, (bf16_t*)vc, P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,  \
-        tile_entry, tile_row0, n_q, n_kv, d, scale, window, softcap, splits, ws, fz, out_tiles, cnt, log2p, pieces)
+        tile_entry, tile_row0, n_q, n_kv, d, scale, window, softcap, splits, ws, fz, out_tiles, cnt, log2p, pieces, dist, sink)
 #define ATT_CASE(DM)                                                                                                          \
     if (qkv && P <= 32) ATT_LAUNCH(DM, true, FULL_STREAMED); else if (qkv) ATT_LAUNCH(DM, true, FULL_KEPT);                      \
     else if (d == DM && P <= 32) ATT_LAUNCH(DM, false, FULL_STREAMED); else if (d == DM) ATT_LAUNCH(DM, false, FULL_KEPT);       \

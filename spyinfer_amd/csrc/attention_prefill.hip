@@ -37,7 +37,11 @@ __global__ __launch_bounds__(PF_ROWS / RT * 4, MINW) void attention_prefill_kern
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
-    int n_q, int n_kv, int d, float scale, int window, float softcap, int log2p, int num_tiles, int splits, float* __restrict__ ws, int out_tiles) {
+    int n_q, int n_kv, int d, float scale, int window, float softcap, int log2p, int num_tiles, int splits, float* __restrict__ ws, int out_tiles,
+    const float* __restrict__ dist, int sink) {
+    // dist != null: [2, n_q] float32, a penalty on the distance taken off every (capped) score: dist[h] ln(1 + dist[n_q + h] (pos - key)).
+    // sink: the softmax's denominator holds one more term, e^0, that has no value: in the keys' first part a row's running
+    // maximum starts at 0 with a sum of 1 (in one of the row's four lanes, whose sums are added at the end).
     constexpr int KK = DMAX / 32, DT = DMAX / 16;
     // 16 elements of padding per staged row: the products' 16-byte reads then have no bank conflicts (measured with
     // SQ_LDS_BANK_CONFLICT: 40 % of the LDS cycles with 8, none with 16; the kernel's time follows only by 0-3 %)
@@ -129,6 +133,14 @@ __global__ __launch_bounds__(PF_ROWS / RT * 4, MINW) void attention_prefill_kern
     float m[RT], l[RT];
 #pragma unroll
     for (int t = 0; t < RT; ++t) { m[t] = -INFINITY; l[t] = 0.f; }
+    // the penalty's two numbers of each row's head, kept over the scale as the scores are: d1 ln(1 + d2 x) / scale = dl1 log2(1 + d2 x)
+    float dl1[RT], dl2[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        dl1[t] = dist ? dist[head[t]] * 0.6931471805599453f / scale : 0.f;
+        dl2[t] = dist ? dist[n_q + head[t]] : 0.f;
+        if (sink && part == 0 && row_ok[t]) { m[t] = 0.f; l[t] = g == 0 ? 1.f : 0.f; }
+    }
 
     bf16x8_t pk[NV], pv[NV];
     int kpg[NV], vpg[NV];        // pages of this thread's vectors, looked up one round ahead of the data
@@ -253,6 +265,11 @@ __global__ __launch_bounds__(PF_ROWS / RT * 4, MINW) void attention_prefill_kern
                     // capped scores, cap tanh(score scale / cap), kept over the scale so that what follows is as without a cap
 #pragma unroll
                     for (int j = 0; j < 8; ++j) sc[j] = cap_over_scale * capped_tanh(sc[j] * scale_over_cap);
+                }
+                if (dist) {
+                    const int dist0 = pos[t] - (h0 + 8 * g);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) sc[j] -= dl1[t] * __builtin_amdgcn_logf(fmaf(dl2[t], (float)max(dist0 - j, 0), 1.0f));
                 }
                 if (!unmasked) {
                     // (the empty statement keeps the masks' index arithmetic inside this branch: the compiler had moved
@@ -389,7 +406,8 @@ static long long cu_count() {
 extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, const void* vc, int P, int num_pages, const int* cu_q,
                                      const int* pos0, const int* kv_len, const int* block_table, int max_blocks,
                                      const int* tile_entry, const int* tile_row0, int num_tiles, int tile_rows, int S, int T, int n_q,
-                                     int n_kv, int d, float scale, int window, float softcap, int splits, float* ws, int out_tiles, hipStream_t st) {
+                                     int n_kv, int d, float scale, int window, float softcap, int splits, float* ws, int out_tiles, const float* dist, int sink,
+                                     hipStream_t st) {
     SPY_REQUIRE(num_tiles > 0 && S > 0 && T > 0 && n_q > 0 && n_kv > 0 && num_pages > 0 && max_blocks > 0,
                 "spy_attention_prefill: empty operand");
     SPY_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "spy_attention_prefill: head_dim %d is not a multiple of 16 in 16..128", d);
@@ -410,7 +428,7 @@ extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, c
     const dim3 mgrid(num_tiles * (tile_rows / 16), n_kv);
     const bool one_per_cu = (long long)grid.x * grid.y * grid.z <= cu_count();
 #define PF_ARGS (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, P, num_pages, cu_q, pos0, kv_len, block_table,   \
-                max_blocks, tile_entry, tile_row0, n_q, n_kv, d, scale, window, softcap, log2p, num_tiles, splits, ws, out_tiles
+                max_blocks, tile_entry, tile_row0, n_q, n_kv, d, scale, window, softcap, log2p, num_tiles, splits, ws, out_tiles, dist, sink
     // (head sizes other than 64 and 128 keep the 4-wave shape: with conditions in the head-dim loops the other needs too many registers)
 #define PF_CASE(DM)                                                                                                              \
     if (tile_rows == 256) attention_prefill_kernel<DM, true, 2, 2, 256><<<grid, 512, 0, st>>>(PF_ARGS);                          \

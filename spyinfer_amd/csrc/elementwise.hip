@@ -110,7 +110,12 @@ extern "C" int spy_embedding_sumsq(float* out, void* xw, float* ss, const void* 
 template <typename TA, typename TW, bool VEC>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restrict__ delta, const TA* __restrict__ delta2,
                                    const TW* __restrict__ w, float eps, TA* __restrict__ out, const int* __restrict__ rows, int T,
-                                   int H, int ld, const TA* __restrict__ gate, const TW* __restrict__ gbias, float mult) {
+                                   int H, int ld, const TA* __restrict__ gate, const TW* __restrict__ gbias, float mult,
+                                   const float* __restrict__ base, const float* __restrict__ vec, const TW* __restrict__ w2,
+                                   TA* __restrict__ out2) {
+    // base != null: a float32 addend [T, ld] (an earlier state of the stream that meets it again); vec != null: a float32
+    // vector [ld] added to every row; w2/out2 != null: a second norm of the same sum with a weight of its own (two
+    // sublayers that each read the stream through their own norm).
     // gate != null: the addend is delta * mult * sigmoid(gate + gbias), element by element (a sublayer's result behind its
     // gate), formed here in float32 from the sublayer's result and the gate's product.
     // H: values that are normed together: the whole row (ld == H), or one of the row's ld / H consecutive groups, which
@@ -132,8 +137,12 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
     TA* o = out + (size_t)r * ld + g0;
     const TA* gt = gate ? gate + (size_t)t * ld + g0 : nullptr;
     const TW* gb = gate ? gbias + g0 : nullptr;
+    const float* bs = base ? base + (size_t)t * ld + g0 : nullptr;
+    const float* vc = vec ? vec + g0 : nullptr;
+    TA* o2 = out2 ? out2 + (size_t)r * ld + g0 : nullptr;
     w += g0;
-    const bool write_back = dl && !rows;
+    if (w2) w2 += g0;
+    const bool write_back = (dl || bs || vc) && !rows;
     if (VEC) {
         // H % 4 == 0 and 16-byte aligned rows (checked by the launcher); the row fits the register passes
         float v[NORM_PASSES][4];
@@ -162,6 +171,18 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[p][e] += d4[e];
                 }
+                if (bs) {
+                    float b4[4];
+                    Vec4<float>::load(bs + i, b4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[p][e] += b4[e];
+                }
+                if (vc) {
+                    float c4[4];
+                    Vec4<float>::load(vc + i, c4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[p][e] += c4[e];
+                }
                 if (write_back) Vec4<float>::store(x + i, v[p]);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) ss += v[p][e] * v[p][e];
@@ -178,6 +199,12 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
 #pragma unroll
                 for (int e = 0; e < 4; ++e) y[e] = (scale * v[p][e]) * w4[e];
                 Vec4<TA>::store(o + i, y);
+                if (o2) {
+                    Vec4<TW>::load(w2 + i, w4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) y[e] = (scale * v[p][e]) * w4[e];
+                    Vec4<TA>::store(o2 + i, y);
+                }
             }
         }
         return;
@@ -190,6 +217,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
             if (gt) a = a * mult / (1.0f + expf(-(to_f32<TA>(gt[i]) + to_f32<TW>(gb[i]))));
             v += a;
         }
+        if (bs) v += bs[i];
+        if (vc) v += vc[i];
         if (write_back) x[i] = v;
         ss += v * v;
     }
@@ -202,14 +231,20 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
             if (gt) a = a * mult / (1.0f + expf(-(to_f32<TA>(gt[i]) + to_f32<TW>(gb[i]))));
             v += a;
         }
+        if (rows) {
+            if (bs) v += bs[i];
+            if (vc) v += vc[i];
+        }
         o[i] = from_f32<TA>((scale * v) * to_f32<TW>(w[i]));
+        if (o2) o2[i] = from_f32<TA>((scale * v) * to_f32<TW>(w2[i]));
     }
 }
 
 extern "C" int spy_add_rmsnorm(float* resid, const void* delta, const void* delta2, const void* w, int w_dtype, float eps, void* out,
                                int out_dtype, const int* rows, int n_out, int T, int ld, int groups, const void* gate, const void* gbias,
-                               float mult, hipStream_t st) {
+                               float mult, const float* base, const float* vec, const void* w2, void* out2, hipStream_t st) {
     SPY_REQUIRE(n_out > 0 && T > 0 && ld > 0, "spy_add_rmsnorm: empty operand");
+    SPY_REQUIRE((w2 == nullptr) == (out2 == nullptr), "spy_add_rmsnorm: a second norm needs its weight and its output");
     SPY_REQUIRE(!gate || (delta && gbias), "spy_add_rmsnorm: a gate without an addend or without its bias");
     SPY_REQUIRE(groups > 0 && groups <= 65535 && ld % groups == 0, "spy_add_rmsnorm: %d groups do not divide rows of %d", groups, ld);
     SPY_REQUIRE(delta || !delta2, "spy_add_rmsnorm: a second addend without a first");
@@ -217,23 +252,27 @@ extern "C" int spy_add_rmsnorm(float* resid, const void* delta, const void* delt
     const dim3 grid(n_out, groups);
     const int threads = H >= 2048 ? 256 : (H >= 512 ? 128 : 64);
     const bool aligned = H % 4 == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)delta % 16) == 0 && ((uintptr_t)delta2 % 16) == 0 && ((uintptr_t)w % 16) == 0 &&
-                         ((uintptr_t)out % 16) == 0 && ((uintptr_t)gate % 16) == 0 && ((uintptr_t)gbias % 16) == 0;
-    const bool vec = aligned && H <= threads * 4 * NORM_PASSES;
-    if (vec) {
+                         ((uintptr_t)out % 16) == 0 && ((uintptr_t)gate % 16) == 0 && ((uintptr_t)gbias % 16) == 0 &&
+                         ((uintptr_t)base % 16) == 0 && ((uintptr_t)vec % 16) == 0 && ((uintptr_t)w2 % 16) == 0 && ((uintptr_t)out2 % 16) == 0;
+    const bool by_pieces = aligned && H <= threads * 4 * NORM_PASSES;
+    if (by_pieces) {
         SPY_DISPATCH(out_dtype, TA, SPY_DISPATCH(w_dtype, TW, (add_rmsnorm_kernel<TA, TW, true><<<grid, threads, 0, st>>>(
-            resid, (const TA*)delta, (const TA*)delta2, (const TW*)w, eps, (TA*)out, rows, T, H, ld, (const TA*)gate, (const TW*)gbias, mult))));
+            resid, (const TA*)delta, (const TA*)delta2, (const TW*)w, eps, (TA*)out, rows, T, H, ld, (const TA*)gate, (const TW*)gbias, mult,
+            base, vec, (const TW*)w2, (TA*)out2))));
     } else {
         SPY_DISPATCH(out_dtype, TA, SPY_DISPATCH(w_dtype, TW, (add_rmsnorm_kernel<TA, TW, false><<<grid, 512, 0, st>>>(
-            resid, (const TA*)delta, (const TA*)delta2, (const TW*)w, eps, (TA*)out, rows, T, H, ld, (const TA*)gate, (const TW*)gbias, mult))));
+            resid, (const TA*)delta, (const TA*)delta2, (const TW*)w, eps, (TA*)out, rows, T, H, ld, (const TA*)gate, (const TW*)gbias, mult,
+            base, vec, (const TW*)w2, (TA*)out2))));
     }
     SPY_CHECK_LAUNCH("spy_add_rmsnorm");
     return 0;
 }
 
 template <typename TA, typename TW>
-__global__ void rmsnorm_kernel(const TA* __restrict__ x, const TW* __restrict__ w, float eps, TA* __restrict__ out, int n) {
+__global__ void rmsnorm_kernel(const TA* __restrict__ x, long long ldx, const TW* __restrict__ w, float eps, TA* __restrict__ out, int n) {
+    // (ldx: values from one input row to the next: the rows may lie inside a wider product; the output is dense)
     __shared__ float red[16];
-    const TA* xr = x + (size_t)blockIdx.x * n;
+    const TA* xr = x + (size_t)blockIdx.x * ldx;
     float ss = 0.f;
     for (int i = threadIdx.x; i < n; i += blockDim.x) { float v = to_f32<TA>(xr[i]); ss += v * v; }
     ss = block_sum(ss, red);
@@ -242,13 +281,30 @@ __global__ void rmsnorm_kernel(const TA* __restrict__ x, const TW* __restrict__ 
     for (int i = threadIdx.x; i < n; i += blockDim.x) o[i] = from_f32<TA>((scale * to_f32<TA>(xr[i])) * to_f32<TW>(w[i]));
 }
 
-extern "C" int spy_rmsnorm(const void* x, int x_dtype, const void* w, int w_dtype, float eps, void* out, int64_t rows, int n,
+extern "C" int spy_rmsnorm(const void* x, long long ldx, int x_dtype, const void* w, int w_dtype, float eps, void* out, int64_t rows, int n,
                            hipStream_t st) {
-    SPY_REQUIRE(rows > 0 && rows < (1ll << 31) && n > 0, "spy_rmsnorm: bad sizes");
+    SPY_REQUIRE(rows > 0 && rows < (1ll << 31) && n > 0 && ldx >= n, "spy_rmsnorm: bad sizes");
     const int threads = n >= 1024 ? 512 : (n > 64 ? 256 : 64);
     SPY_DISPATCH(x_dtype, TA, SPY_DISPATCH(w_dtype, TW, (rmsnorm_kernel<TA, TW><<<(unsigned)rows, threads, 0, st>>>(
-        (const TA*)x, (const TW*)w, eps, (TA*)out, n))));
+        (const TA*)x, ldx, (const TW*)w, eps, (TA*)out, n))));
     SPY_CHECK_LAUNCH("spy_rmsnorm");
+    return 0;
+}
+
+// x[i] = cap tanh(x[i] scale / cap) in place over float32 values (cap == 0: x[i] * scale): logits behind their head
+__global__ void scale_cap_kernel(float* __restrict__ x, size_t n, float scale, float cap) {
+    const float inv = cap > 0.f ? 1.0f / cap : 0.f;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const float v = x[i] * scale;
+        x[i] = cap > 0.f ? cap * tanhf(v * inv) : v;
+    }
+}
+
+extern "C" int spy_scale_cap(float* x, int64_t n, float scale, float cap, hipStream_t st) {
+    SPY_REQUIRE(n > 0 && cap >= 0.f, "spy_scale_cap: bad sizes");
+    const unsigned blocks = (unsigned)((n + 255) / 256 > 65536 ? 65536 : (n + 255) / 256);
+    scale_cap_kernel<<<blocks, 256, 0, st>>>(x, (size_t)n, scale, cap);
+    SPY_CHECK_LAUNCH("spy_scale_cap");
     return 0;
 }
 

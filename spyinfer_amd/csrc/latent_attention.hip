@@ -22,7 +22,8 @@ template <typename TA, typename TW, typename TQ>
 __global__ void latent_prepare_kernel(TQ* __restrict__ qa, const TA* __restrict__ q, int ldq, const TA* __restrict__ dkv, int ldd,
                                       TA* __restrict__ cache, const int* __restrict__ slot_mapping, long long cache_rows,
                                       const TW* __restrict__ w_norm, float eps, const float* __restrict__ freq, float mag,
-                                      int dims, const int* __restrict__ positions, int H, int DN, int DR, int R) {
+                                      int dims, const int* __restrict__ positions, int H, int DN, int DR, int R, int interleaved) {
+    // interleaved: pair j of the rotated dims is (2 j, 2 j + 1) instead of (j, j + dims / 2)
     __shared__ float red[16];
     __shared__ float cs[LP_MAX_PAIRS], sn[LP_MAX_PAIRS];
     const int t = blockIdx.x;
@@ -41,9 +42,10 @@ __global__ void latent_prepare_kernel(TQ* __restrict__ qa, const TA* __restrict_
         const TA* src = q + (size_t)t * ldq + (size_t)h * (DN + DR) + DN;
         float v = to_f32<TA>(src[i]);
         if (i < dims) {
-            const int j = i < half ? i : i - half;
-            const float a = to_f32<TA>(src[j]), b = to_f32<TA>(src[j + half]);
-            v = i < half ? a * cs[j] - b * sn[j] : b * cs[j] + a * sn[j];
+            const bool first = interleaved ? !(i & 1) : i < half;
+            const int j = interleaved ? i >> 1 : (i < half ? i : i - half);
+            const float a = to_f32<TA>(src[interleaved ? 2 * j : j]), b = to_f32<TA>(src[interleaved ? 2 * j + 1 : j + half]);
+            v = first ? a * cs[j] - b * sn[j] : b * cs[j] + a * sn[j];
         }
         qa[((size_t)t * H + h) * (R + DR) + R + i] = from_f32<TQ>(v);
     }
@@ -60,9 +62,10 @@ __global__ void latent_prepare_kernel(TQ* __restrict__ qa, const TA* __restrict_
     for (int i = threadIdx.x; i < DR; i += blockDim.x) {
         float v = to_f32<TA>(d[R + i]);
         if (i < dims) {
-            const int j = i < half ? i : i - half;
-            const float a = to_f32<TA>(d[R + j]), b = to_f32<TA>(d[R + j + half]);
-            v = i < half ? a * cs[j] - b * sn[j] : b * cs[j] + a * sn[j];
+            const bool first = interleaved ? !(i & 1) : i < half;
+            const int j = interleaved ? i >> 1 : (i < half ? i : i - half);
+            const float a = to_f32<TA>(d[R + (interleaved ? 2 * j : j)]), b = to_f32<TA>(d[R + (interleaved ? 2 * j + 1 : j + half)]);
+            v = first ? a * cs[j] - b * sn[j] : b * cs[j] + a * sn[j];
         }
         row[R + i] = from_f32<TA>(v);
     }
@@ -71,14 +74,14 @@ __global__ void latent_prepare_kernel(TQ* __restrict__ qa, const TA* __restrict_
 extern "C" int spy_latent_prepare(void* qa, int qa_dtype, const void* q, int ldq, const void* dkv, int ldd, int dtype, void* cache,
                                   const int* slot_mapping, long long cache_rows, const void* w_norm, int w_dtype, float eps,
                                   const float* freq, float mag, int dims, const int* positions, int T, int H, int DN, int DR, int R,
-                                  hipStream_t st) {
+                                  int interleaved, hipStream_t st) {
     SPY_REQUIRE(T > 0 && H > 0 && DN >= 0 && DR >= 0 && R > 0, "spy_latent_prepare: empty operand");
     SPY_REQUIRE(dims >= 0 && dims <= DR && dims % 2 == 0 && (dims == 0 || freq) && dims / 2 <= LP_MAX_PAIRS,
                 "spy_latent_prepare: %d rotated dims of %d (an even number up to %d)", dims, DR, 2 * LP_MAX_PAIRS);
     SPY_REQUIRE(!dkv || (cache && slot_mapping && w_norm), "spy_latent_prepare: storing needs the cache, the tokens' slots and the norm weight");
     SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, SPY_DISPATCH(qa_dtype, TQ, (latent_prepare_kernel<TA, TW, TQ><<<T, 256, 0, st>>>(
         (TQ*)qa, (const TA*)q, ldq, (const TA*)dkv, ldd, (TA*)cache, slot_mapping, cache_rows, (const TW*)w_norm, eps, freq, mag, dims,
-        positions, H, DN, DR, R)))));
+        positions, H, DN, DR, R, interleaved)))));
     SPY_CHECK_LAUNCH("spy_latent_prepare");
     return 0;
 }

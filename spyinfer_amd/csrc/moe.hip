@@ -33,11 +33,18 @@ __device__ __forceinline__ float moe_gated(float g, float u, const MoeAct& a, fl
 // one wave per token
 __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ ids, float* __restrict__ weights, const float* __restrict__ z,
                                                        const float* __restrict__ correction, int E, int top, int groups, int keep,
-                                                       float scale, int sigmoid, int renorm) {
+                                                       float scale, int sigmoid, int renorm, const float* __restrict__ zbias) {
+    // zbias != null: a bias [E] that is part of the logits (it moves the scores and with them the weights, where the
+    // correction moves the choice alone)
     __shared__ float sc[MOE_MAX_EXPERTS], ch[MOE_MAX_EXPERTS], gsc[MOE_MAX_EXPERTS];
+    __shared__ float zb[MOE_MAX_EXPERTS];
     __shared__ int allowed[MOE_MAX_EXPERTS], sel[MOE_MAX_EXPERTS];
     const int t = blockIdx.x, lane = threadIdx.x;
     const float* zr = z + (size_t)t * E;
+    if (zbias) {
+        for (int e = lane; e < E; e += 64) zb[e] = zr[e] + zbias[e];     // (a lane reads back only what it wrote: no barrier)
+        zr = zb;
+    }
     if (sigmoid) {
         // every logit by itself
         for (int e = lane; e < E; e += 64) {
@@ -112,11 +119,11 @@ __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ ids, fl
 }
 
 extern "C" int spy_moe_route(int* ids, float* weights, const float* z, const float* correction, int T, int E, int top, int groups,
-                             int keep, float scale, int sigmoid, int renorm, hipStream_t st) {
+                             int keep, float scale, int sigmoid, int renorm, const float* zbias, hipStream_t st) {
     SPY_REQUIRE(T > 0 && E > 0 && E <= MOE_MAX_EXPERTS, "spy_moe_route: %d experts (1..%d)", E, MOE_MAX_EXPERTS);
     SPY_REQUIRE(groups > 0 && E % groups == 0 && keep > 0 && keep <= groups && top > 0 && top <= keep * (E / groups),
                 "spy_moe_route: %d of %d groups of %d experts cannot give %d choices", keep, groups, E / (groups > 0 ? groups : 1), top);
-    moe_route_kernel<<<T, 64, 0, st>>>(ids, weights, z, correction, E, top, groups, keep, scale, sigmoid, renorm);
+    moe_route_kernel<<<T, 64, 0, st>>>(ids, weights, z, correction, E, top, groups, keep, scale, sigmoid, renorm, zbias);
     SPY_CHECK_LAUNCH("spy_moe_route");
     return 0;
 }
@@ -521,10 +528,11 @@ extern "C" int spy_moe_gemm(void* C, int c_dtype, const void* A, int a_dtype, co
     return 0;
 }
 
-// out[t, :] = sum_k weights[t, k] * Y[pair_row[t top + k], :], added in ascending k (no weights: all one)
+// out[t, :] = sum_k weights[t, k] * Y[pair_row[t top + k], :], added in ascending k (no weights: all one); add != null:
+// plus add[t, :], the result of a layer that every token uses, in the same pass
 template <typename TC>
 __global__ void moe_combine_kernel(TC* __restrict__ out, const float* __restrict__ Y, const float* __restrict__ weights,
-                                   const int* __restrict__ pair_row, int top, int H) {
+                                   const int* __restrict__ pair_row, int top, int H, const TC* __restrict__ add) {
     const int t = blockIdx.x;
     for (int c = threadIdx.x; c < H; c += blockDim.x) {
         float acc = 0.f;
@@ -532,14 +540,15 @@ __global__ void moe_combine_kernel(TC* __restrict__ out, const float* __restrict
             const int row = pair_row[(size_t)t * top + k];
             if (row >= 0) acc = fmaf(weights ? weights[(size_t)t * top + k] : 1.f, Y[(size_t)row * H + c], acc);
         }
+        if (add) acc += to_f32<TC>(add[(size_t)t * H + c]);
         out[(size_t)t * H + c] = from_f32<TC>(acc);
     }
 }
 
 extern "C" int spy_moe_combine(void* out, int dtype, const float* Y, const float* weights, const int* pair_row, int T, int top, int H,
-                               hipStream_t st) {
+                               const void* add, hipStream_t st) {
     SPY_REQUIRE(T > 0 && top > 0 && H > 0, "spy_moe_combine: empty operand");
-    SPY_DISPATCH(dtype, TC, (moe_combine_kernel<TC><<<T, 256, 0, st>>>((TC*)out, Y, weights, pair_row, top, H)));
+    SPY_DISPATCH(dtype, TC, (moe_combine_kernel<TC><<<T, 256, 0, st>>>((TC*)out, Y, weights, pair_row, top, H, (const TC*)add)));
     SPY_CHECK_LAUNCH("spy_moe_combine");
     return 0;
 }

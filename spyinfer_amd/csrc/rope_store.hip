@@ -16,7 +16,9 @@ template <typename TA, typename TW>
 __global__ __launch_bounds__(RS_WAVES * 64) void bias_rope_store_kernel(
     const TA* __restrict__ x, long long xs, TA* __restrict__ q_out, int n_q, int n_kv, int d, const TW* __restrict__ bias,
     const float* __restrict__ freq, int rot, const int* __restrict__ positions, TA* __restrict__ kc, TA* __restrict__ vc, int P,
-    int num_pages, const int* __restrict__ slots, float mag, float v_eps, int v_n) {
+    int num_pages, const int* __restrict__ slots, float mag, float v_eps, int v_n, float qt_coef, int qt_every) {
+    // qt_every > 0: a query is multiplied by 1 + qt_coef ln(floor((position + 1) / qt_every) + 1), float32 (queries that grow
+    // with the logarithm of the position, in steps of qt_every positions)
     const int t = blockIdx.x, lane = threadIdx.x & 63;
     const int h = blockIdx.y * RS_WAVES + (threadIdx.x >> 6);
     const int heads = n_q + 2 * n_kv;
@@ -50,21 +52,23 @@ __global__ __launch_bounds__(RS_WAVES * 64) void bias_rope_store_kernel(
     }
     const int half = rot >> 1;
     const float p = (float)positions[t];
+    const float qt = (is_q && qt_every > 0) ? 1.0f + qt_coef * logf((float)((positions[t] + 1) / qt_every) + 1.0f) : 1.0f;
     TA* dst = is_q ? q_out + ((size_t)t * n_q + h) * d : kc + (((size_t)page * n_kv + (h - n_q)) * P + off) * d;
     for (int j = lane; j < half; j += 64) {
         const float a = to_f32<TA>(row[j]) + (b ? to_f32<TW>(b[j]) : 0.f);
         const float c = to_f32<TA>(row[j + half]) + (b ? to_f32<TW>(b[j + half]) : 0.f);
         const float ang = p * freq[j];
         const float cs = cosf(ang) * mag, sn = sinf(ang) * mag;
-        dst[j] = from_f32<TA>(a * cs - c * sn);
-        dst[j + half] = from_f32<TA>(c * cs + a * sn);
+        dst[j] = from_f32<TA>((a * cs - c * sn) * qt);
+        dst[j + half] = from_f32<TA>((c * cs + a * sn) * qt);
     }
-    for (int j = rot + lane; j < d; j += 64) dst[j] = from_f32<TA>(to_f32<TA>(row[j]) + (b ? to_f32<TW>(b[j]) : 0.f));
+    for (int j = rot + lane; j < d; j += 64) dst[j] = from_f32<TA>((to_f32<TA>(row[j]) + (b ? to_f32<TW>(b[j]) : 0.f)) * qt);
 }
 
 extern "C" int spy_bias_rope_store(const void* x, long long xs, int dtype, void* q_out, int T, int n_q, int n_kv, int d,
                                    const void* bias, int b_dtype, const float* freq, int rot, const int* positions, void* kc,
-                                   void* vc, int P, int num_pages, const int* slots, float mag, float v_eps, int v_n, hipStream_t st) {
+                                   void* vc, int P, int num_pages, const int* slots, float mag, float v_eps, int v_n, float qt_coef, int qt_every,
+                                   hipStream_t st) {
     SPY_REQUIRE(T > 0 && n_q > 0 && n_kv > 0 && d > 0 && xs >= (long long)(n_q + 2 * n_kv) * d, "spy_bias_rope_store: bad sizes");
     SPY_REQUIRE(d <= RS_MAX_D, "spy_bias_rope_store: head size %d exceeds the supported %d", d, RS_MAX_D);
     SPY_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0 && (rot == 0 || freq), "spy_bias_rope_store: %d rotated dims do not fit a head of %d", rot, d);
@@ -73,31 +77,34 @@ extern "C" int spy_bias_rope_store(const void* x, long long xs, int dtype, void*
     SPY_REQUIRE(v_n >= 0 && v_n <= d, "spy_bias_rope_store: a value norm over %d of %d values", v_n, d);
     const dim3 grid(T, (n_q + 2 * n_kv + RS_WAVES - 1) / RS_WAVES);
     SPY_DISPATCH(dtype, TA, SPY_DISPATCH(b_dtype, TW, (bias_rope_store_kernel<TA, TW><<<grid, RS_WAVES * 64, 0, st>>>(
-        (const TA*)x, xs, (TA*)q_out, n_q, n_kv, d, (const TW*)bias, freq, rot, positions, (TA*)kc, (TA*)vc, P, num_pages, slots, mag, v_eps, v_n))));
+        (const TA*)x, xs, (TA*)q_out, n_q, n_kv, d, (const TW*)bias, freq, rot, positions, (TA*)kc, (TA*)vc, P, num_pages, slots, mag, v_eps, v_n,
+        qt_coef, qt_every))));
     SPY_CHECK_LAUNCH("spy_bias_rope_store");
     return 0;
 }
 
-// y[t, j] *= mult * sigmoid(g[t, j] + bias[j]) in place; the gate's rows may be part of a wider product (`gs` values from
-// row to row); the bias may be absent.
+// y[t, j] *= mult * sigmoid(g[t, j / per] + bias[j / per]) in place; the gate's rows may be part of a wider product (`gs`
+// values from row to row); the bias may be absent.  per: columns of y that share one gate value (1: a gate per column;
+// a head's size: one number per head).
 template <typename TA, typename TW>
 __global__ void sigmoid_gate_kernel(TA* __restrict__ y, const TA* __restrict__ g, long long gs, const TW* __restrict__ bias, float mult,
-                                    int T, int N) {
+                                    int T, int N, int per) {
     const size_t total = (size_t)T * N;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const size_t t = i / N, j = i - t * N;
-        const float gate = to_f32<TA>(g[t * gs + j]) + (bias ? to_f32<TW>(bias[j]) : 0.f);
+        const size_t c = per > 1 ? j / per : j;
+        const float gate = to_f32<TA>(g[t * gs + c]) + (bias ? to_f32<TW>(bias[c]) : 0.f);
         y[i] = from_f32<TA>(to_f32<TA>(y[i]) * mult / (1.0f + expf(-gate)));
     }
 }
 
 extern "C" int spy_sigmoid_gate(void* y, const void* g, long long gs, int dtype, const void* bias, int b_dtype, float mult, int T, int N,
-                                hipStream_t st) {
-    SPY_REQUIRE(T > 0 && N > 0 && gs >= N, "spy_sigmoid_gate: bad sizes");
+                                int per, hipStream_t st) {
+    SPY_REQUIRE(T > 0 && N > 0 && per > 0 && N % per == 0 && gs >= N / per, "spy_sigmoid_gate: bad sizes");
     const size_t total = (size_t)T * N;
     const unsigned blocks = (unsigned)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256);
     SPY_DISPATCH(dtype, TA, SPY_DISPATCH(b_dtype, TW, (sigmoid_gate_kernel<TA, TW><<<blocks, 256, 0, st>>>((TA*)y, (const TA*)g, gs,
-        (const TW*)bias, mult, T, N))));
+        (const TW*)bias, mult, T, N, per))));
     SPY_CHECK_LAUNCH("spy_sigmoid_gate");
     return 0;
 }

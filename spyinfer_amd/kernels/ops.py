@@ -79,7 +79,7 @@ class _Hip:
                      "spy_gemm_strided", "spy_latent_attention", "spy_latent_attention_mfma", "spy_latent_attention_mfma_workspace", "spy_head_products",
                      "spy_bias_rope_store", "spy_sigmoid_gate", "spy_mlstm", "spy_causal_conv_silu", "spy_delta_rule", "spy_moe_route",
                      "spy_moe_align", "spy_moe_gemm", "spy_moe_combine", "spy_moe_tile_rows", "spy_token_shift", "spy_tanh", "spy_time_mix",
-                     "spy_norm_pair_mean"):
+                     "spy_norm_pair_mean", "spy_scale_cap"):
             if not hasattr(self.lib, name):
                 raise KernelError("the kernel library %s lacks %s: it is older than its sources; build it again "
                                   "(spyinfer_amd.kernels.build.build())" % (self.lib._name, name))
@@ -138,11 +138,14 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> tor
 
 def add_rms_norm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
                  out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None, delta2: Optional[torch.Tensor] = None, groups: int = 1,
-                 gate=None) -> torch.Tensor:
+                 gate=None, base: Optional[torch.Tensor] = None, vec: Optional[torch.Tensor] = None,
+                 weight2: Optional[torch.Tensor] = None):
     """resid += delta (float32, in place; skipped if delta is None), then RMS-normalise.  ``delta2``: a second addend
     (two sublayers that read one norm): resid += delta + delta2, the two summed in float32 first.  ``groups``: the row is
     cut into that many equal consecutive parts, each over its own root mean square.  ``gate`` = (rows [T, H] of the activation
     dtype, bias [H] of the weight's dtype, constant): the addend is delta * constant * sigmoid(rows + bias), formed in float32.
+    ``base``: a float32 addend [T, H] (an earlier state of the stream); ``vec``: a float32 vector [H] added to every row.
+    ``weight2``: a second norm of the same sum with this weight: the result is then the pair of both outputs.
 
     Without ``rows``: every row is updated and normalised -> [T, H].  With ``rows``
     (int32 [R]): only those rows are summed and normalised -> [R, H]; resid is left as it is."""
@@ -162,26 +165,48 @@ def add_rms_norm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: tor
         _dev(g_rows, g_bias)
         _check(delta is not None and g_rows.shape == (T, H) and g_rows.dtype == out_dtype and g_bias.shape == (H,) and g_bias.dtype == weight.dtype,
                "add_rms_norm: the gate's rows must be like the addend and its bias like the norm's weight")
+    _dev(base, vec, weight2)
+    _check(base is None or (base.shape == (T, H) and base.dtype == torch.float32 and base.is_contiguous()),
+           "add_rms_norm: the float32 addend must be [T, H]")
+    _check(vec is None or (vec.shape == (H,) and vec.dtype == torch.float32 and vec.is_contiguous()), "add_rms_norm: the row vector must be float32 [H]")
+    _check(weight2 is None or (weight2.shape == (H,) and weight2.dtype == weight.dtype), "add_rms_norm: the second weight must be like the first")
     n_out = T if rows is None else rows.shape[0]
     out = torch.empty((n_out, H), dtype=out_dtype, device=resid.device)
+    out2 = torch.empty_like(out) if weight2 is not None else None
     if n_out:
         hip().call("spy_add_rmsnorm", _ptr(resid), _ptr(delta), _ptr(delta2), _ptr(weight), _code(weight, "norm weight"),
                    ctypes.c_float(eps), _ptr(out), _code(out, "norm output"), _ptr(rows), ctypes.c_int(n_out),
-                   ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(groups), _ptr(g_rows), _ptr(g_bias), ctypes.c_float(g_mult), _Hip.stream())
-    return out
+                   ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(groups), _ptr(g_rows), _ptr(g_bias), ctypes.c_float(g_mult),
+                   _ptr(base), _ptr(vec), _ptr(weight2), _ptr(out2), _Hip.stream())
+    return out if weight2 is None else (out, out2)
 
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
-    """RMS norm over the last dimension, same dtype out as in."""
+    """RMS norm over the last dimension, same dtype out as in.  A two-dimensional ``x`` may be a view into the rows of a
+    wider product (its row stride is taken); the result is dense."""
     _dev(x, weight)
     n = x.shape[-1]
     _check(weight.shape == (n,), "rms_norm: weight must match the last dimension")
-    out = torch.empty_like(x)
+    ldx = n
+    if x.dim() == 2 and x.stride(1) == 1 and x.stride(0) >= n:
+        ldx = x.stride(0)
+    else:
+        _check(x.is_contiguous(), "rms_norm: dense input, or rows of a wider product, expected")
+    out = torch.empty(tuple(x.shape), dtype=x.dtype, device=x.device)
     rows = x.numel() // n if n else 0
     if rows:
-        hip().call("spy_rmsnorm", _ptr(x), _code(x, "rms_norm input"), _ptr(weight), _code(weight, "norm weight"),
-                   ctypes.c_float(eps), _ptr(out), ctypes.c_int64(rows), ctypes.c_int(n), _Hip.stream())
+        hip().call("spy_rmsnorm", ctypes.c_void_p(x.data_ptr()), ctypes.c_longlong(ldx), _code(x, "rms_norm input"), _ptr(weight),
+                   _code(weight, "norm weight"), ctypes.c_float(eps), _ptr(out), ctypes.c_int64(rows), ctypes.c_int(n), _Hip.stream())
     return out
+
+
+def scale_cap(x: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> torch.Tensor:
+    """In place over float32 values: x = cap tanh(x scale / cap) (``cap`` 0: x * scale): logits behind their head."""
+    _dev(x)
+    _check(x.dtype == torch.float32 and x.is_contiguous() and cap >= 0.0, "scale_cap: dense float32 values and a cap >= 0 expected")
+    if x.numel() and (scale != 1.0 or cap > 0.0):
+        hip().call("spy_scale_cap", _ptr(x), ctypes.c_int64(x.numel()), ctypes.c_float(scale), ctypes.c_float(cap), _Hip.stream())
+    return x
 
 
 #: A bfloat16 product with at most this many rows runs on the hand-written streaming MFMA kernel
@@ -416,6 +441,28 @@ class GatedAddend:
 
     def resolve(self):
         return sigmoid_gate(self.y, self.gate, self.bias, self.mult)
+
+
+class EntryAddends:
+    """What meets the stream where a walk over a run of layers begins: whatever the block before left pending (None, an
+    addend, a pair of addends), an earlier state of the stream (``base``, float32 [T, H], or None) and a vector that
+    every row gets (``vec``, float32 [H]).  The norm that reads the stream next sums all of it in its kernel's pass."""
+
+    __slots__ = ("pending", "base", "vec")
+
+    def __init__(self, pending, base, vec):
+        self.pending, self.base, self.vec = pending, base, vec
+
+    def resolve(self, resid: torch.Tensor) -> None:
+        """Sums everything into the stream with plain tensor operations (for a reader that has no kernel for it)."""
+        pend = None if isinstance(self.pending, ScaledInput) else self.pending
+        for addend in (pend if isinstance(pend, (tuple, list)) else (pend,)):
+            if addend is not None:
+                resid.add_((addend.resolve() if isinstance(addend, GatedAddend) else addend).float())
+        if self.base is not None:
+            resid.add_(self.base)
+        if self.vec is not None:
+            resid.add_(self.vec)
 
 
 class ScaledInput:
@@ -753,11 +800,13 @@ def fused_attention_ok(dtype, meta: AttentionMeta, n_q: int, n_kv: int, d: int, 
 
 def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: torch.Tensor, page_size: int, meta: AttentionMeta,
                     n_q: int, n_kv: int, d: int, scale: float, window: Optional[int], raw: Optional[RawQKV] = None,
-                    for_product: bool = False, softcap: float = 0.0):
+                    for_product: bool = False, softcap: float = 0.0, distance: Optional[torch.Tensor] = None, zero_sink: bool = False):
     """Causal grouped-query attention of the step's query tokens over the paged cache
     (which already holds this step's keys and values, or gets them from ``raw`` in this call).  Query at position p
     reads keys max(0, p - window + 1) .. p.  Scores, softmax and the weighted sum are float32.  ``softcap`` > 0: a
-    score is softcap tanh(q . k scale / softcap).
+    score is softcap tanh(q . k scale / softcap).  ``distance``: float32 [2, n_q]: head h's (capped) score of a key that lies
+    x positions back is lowered by distance[0, h] ln(1 + distance[1, h] x).  ``zero_sink``: the softmax's denominator
+    holds one more term, e^0, that has no value: p_j = e^(s_j) / (1 + sum e^(s_j)).
     ``for_product``: the result goes into a decode product only and may come as OperandRows (it does for steps of at
     most 128 tokens, ``attention_hands_over_operand_rows``)."""
     T, S = meta.T, meta.S
@@ -791,6 +840,11 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
     _check(win >= 0, "paged_attention: window must be positive")
     softcap = float(softcap or 0.0)
     _check(softcap >= 0.0 and (raw is None or softcap == 0.0), "paged_attention: the scores' cap must not be negative (and the raw product takes none)")
+    _dev(distance)
+    _check(distance is None or (distance.dtype == torch.float32 and tuple(distance.shape) == (2, n_q) and distance.is_contiguous()),
+           "paged_attention: the distance penalty's numbers must be float32 [2, n_q]")
+    _check(raw is None or (distance is None and not zero_sink), "paged_attention: the raw product takes neither a distance penalty nor a sink")
+    extras = (_ptr(distance), ctypes.c_int(1 if zero_sink else 0))
     out = q if raw is not None else torch.empty_like(q)
     if T == 0:
         return out
@@ -824,7 +878,7 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
             bws = torch.empty((max(1, bws_floats),), dtype=torch.float32, device=q.device)
             hip().call("spy_attention_prefill", _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), *common, _ptr(big_entry),
                        _ptr(big_row0), ctypes.c_int(n_big), ctypes.c_int(meta.big_rows), *sizes, ctypes.c_int(bsplits), _ptr(bws),
-                       ctypes.c_int(operand.tiles if operand is not None else 0), _Hip.stream())
+                       ctypes.c_int(operand.tiles if operand is not None else 0), *extras, _Hip.stream())
         if n_small:
             # Few 16-row tiles cannot fill the chip by themselves (decoding requests, short portions): their keys are
             # split into parts, each part a block of 4 waves that wants 128 keys at least, and a second kernel merges.
@@ -858,13 +912,13 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
                        _ptr(small_entry), _ptr(small_row0), ctypes.c_int(n_small), *sizes, ctypes.c_int(splits), _ptr(ws), *fused,
                        ctypes.c_int(operand.tiles if operand is not None else 0), _ptr(counters),
                        ctypes.c_int(0 if counters is None else ATTENTION_COUNTERS), _ptr(pieces),
-                       ctypes.c_int(0 if pieces is None else pieces.shape[0]), _Hip.stream())
+                       ctypes.c_int(0 if pieces is None else pieces.shape[0]), *extras, _Hip.stream())
         return operand if operand is not None else out
     hip().call("spy_attention_generic", _ptr(out), _ptr(q), _code(q, "q"), _ptr(k_cache), _ptr(v_cache),
                ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(meta.kv_len), _ptr(meta.block_table),
                ctypes.c_int(meta.max_blocks), _ptr(meta.token_entry), _ptr(meta.positions), ctypes.c_int(S), ctypes.c_int(T),
                ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(d), ctypes.c_float(scale), ctypes.c_int(win), ctypes.c_float(softcap),
-               _Hip.stream())
+               *extras, _Hip.stream())
     return out
 
 
@@ -1044,11 +1098,13 @@ def gemm_strided(a: torch.Tensor, a_strides, b: torch.Tensor, b_strides, c: torc
 
 def latent_prepare(q: torch.Tensor, dkv: Optional[torch.Tensor], cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor],
                    w_norm: Optional[torch.Tensor], eps: float, freq: Optional[torch.Tensor], mag: float, dims: int,
-                   positions: torch.Tensor, H: int, DN: int, DR: int, R: int, qa_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+                   positions: torch.Tensor, H: int, DN: int, DR: int, R: int, qa_dtype: torch.dtype = torch.float32,
+                   interleaved: bool = False) -> torch.Tensor:
     """Queries ``q [T, >= H (DN + DR)]`` (a row may be a view into a wider product: its stride is taken) and, if given,
     ``dkv [T, >= R + DR]``: the latent rmsnorm(dkv[:R]) * w_norm and the rotated dkv[R:] go to ``cache [pages, P, R + DR]``
     at the tokens' slots; returns the absorbed query rows [T, H, R + DR] in ``qa_dtype`` with the rotated part filled in
-    (the first R values of a row are for the caller's product with the keys' expansion matrix)."""
+    (the first R values of a row are for the caller's product with the keys' expansion matrix).  ``interleaved``: pair j of
+    the rotated dims is (2 j, 2 j + 1) instead of (j, j + dims / 2)."""
     _check(q.dim() == 2 and q.stride(1) == 1 and q.is_cuda, "latent_prepare: q must be rows on the GPU")
     T = q.shape[0]
     _check(q.shape[1] >= H * (DN + DR), "latent_prepare: q rows hold %d values, %d heads of %d needed", q.shape[1], H, DN + DR)
@@ -1073,7 +1129,7 @@ def latent_prepare(q: torch.Tensor, dkv: Optional[torch.Tensor], cache: Optional
                    ctypes.c_longlong(rows), _ptr(w_norm if dkv is not None else None),
                    _code(w_norm, "norm weight") if dkv is not None else F32, ctypes.c_float(eps), _ptr(freq), ctypes.c_float(mag),
                    ctypes.c_int(dims), _ptr(positions), ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(DN), ctypes.c_int(DR),
-                   ctypes.c_int(R), _Hip.stream())
+                   ctypes.c_int(R), ctypes.c_int(1 if interleaved else 0), _Hip.stream())
     return qa
 
 
@@ -1177,13 +1233,16 @@ def _row_view(x: torch.Tensor, what: str) -> int:
 
 def bias_rope_store(x: torch.Tensor, n_q: int, n_kv: int, d: int, bias: Optional[torch.Tensor], freq: Optional[torch.Tensor],
                     rotary_dim: int, positions: torch.Tensor, k_cache, v_cache, page_size: int, slots: Optional[torch.Tensor],
-                    mag: float = 1.0, value_norm=None) -> torch.Tensor:
+                    mag: float = 1.0, value_norm=None, query_temperature=None) -> torch.Tensor:
     """From rows ``x [T, >= (n_q + 2 n_kv) d]`` = [q heads | k heads | v heads] (a view into a wider product may be
     given): the biases ``bias [(n_q + 2 n_kv) d]`` added, the first ``rotary_dim`` dims of every q and k head rotated
     (pair (j, j + rotary_dim/2), angle float32(position) * freq[j]), q written to the result [T, n_q d], k and v into
     the cache pages at ``slots`` (skipped when None).  ``mag``: factor on cos and sin.  ``value_norm`` = (eps, n): every
-    value head is divided by sqrt(mean of its first n values squared + eps) before it is stored."""
+    value head is divided by sqrt(mean of its first n values squared + eps) before it is stored.  ``query_temperature`` =
+    (coef, every): the query at position p is multiplied by 1 + coef ln(floor((p + 1) / every) + 1), in float32."""
     xs = _row_view(x, "bias_rope_store")
+    qt_coef, qt_every = (float(query_temperature[0]), int(query_temperature[1])) if query_temperature is not None else (0.0, 0)
+    _check(query_temperature is None or qt_every > 0, "bias_rope_store: the query temperature's step must be positive")
     v_eps, v_n = (float(value_norm[0]), int(value_norm[1])) if value_norm is not None else (0.0, 0)
     _check(0 <= v_n <= d, "bias_rope_store: a value norm over %d of %d values", v_n, d)
     T = x.shape[0]
@@ -1206,20 +1265,23 @@ def bias_rope_store(x: torch.Tensor, n_q: int, n_kv: int, d: int, bias: Optional
                    ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(d), _ptr(bias), _code(bias, "bias") if bias is not None else F32,
                    _ptr(freq), ctypes.c_int(rotary_dim), _ptr(positions), _ptr(k_cache if slots is not None else None),
                    _ptr(v_cache if slots is not None else None), ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(slots),
-                   ctypes.c_float(mag), ctypes.c_float(v_eps), ctypes.c_int(v_n), _Hip.stream())
+                   ctypes.c_float(mag), ctypes.c_float(v_eps), ctypes.c_int(v_n), ctypes.c_float(qt_coef), ctypes.c_int(qt_every), _Hip.stream())
     return q
 
 
-def sigmoid_gate(y: torch.Tensor, gate: torch.Tensor, bias: Optional[torch.Tensor] = None, mult: float = 1.0) -> torch.Tensor:
-    """In place: y[t, j] *= mult * sigmoid(gate[t, j] + bias[j]); ``gate`` may be a view into a wider product."""
+def sigmoid_gate(y: torch.Tensor, gate: torch.Tensor, bias: Optional[torch.Tensor] = None, mult: float = 1.0, per: int = 1) -> torch.Tensor:
+    """In place: y[t, j] *= mult * sigmoid(gate[t, j / per] + bias[j / per]); ``gate`` may be a view into a wider product.
+    ``per``: columns of y that share one gate value (a head's size: one number per head)."""
     _dev(y, bias)
-    _check(bias is None or bias.shape == (y.shape[1],), "sigmoid_gate: one bias per column expected")
+    _check(per >= 1 and y.dim() == 2 and y.shape[1] % per == 0, "sigmoid_gate: %d columns per gate value do not divide the rows", per)
+    _check(bias is None or bias.shape == (y.shape[1] // per,), "sigmoid_gate: one bias per gate value expected")
     gs = _row_view(gate, "sigmoid_gate")
-    _check(y.dim() == 2 and gate.shape == y.shape and gate.dtype == y.dtype and gate.device == y.device, "sigmoid_gate: gate rows like y expected")
+    _check(y.is_contiguous() and tuple(gate.shape) == (y.shape[0], y.shape[1] // per) and gate.dtype == y.dtype and gate.device == y.device,
+           "sigmoid_gate: gate rows like y expected")
     if y.numel():
         hip().call("spy_sigmoid_gate", _ptr(y), ctypes.c_void_p(gate.data_ptr()), ctypes.c_longlong(gs), _code(y, "y"), _ptr(bias),
                    _code(bias, "bias") if bias is not None else F32, ctypes.c_float(mult), ctypes.c_int(y.shape[0]), ctypes.c_int(y.shape[1]),
-                   _Hip.stream())
+                   ctypes.c_int(per), _Hip.stream())
     return y
 
 
@@ -1416,12 +1478,15 @@ def norm_pair_mean(a: torch.Tensor, b: torch.Tensor, wa: torch.Tensor, wb: torch
 # --------------------------------------------------------------------------
 # Mixture of experts
 def moe_route(z: torch.Tensor, correction: Optional[torch.Tensor], top: int, groups: int, keep: int, scale: float, score: str = "softmax",
-              renormalize: bool = True):
+              renormalize: bool = True, logit_bias: Optional[torch.Tensor] = None):
     """Router logits ``z [T, E]`` float32 -> (experts int32 [T, top], weights float32 [T, top]): s = softmax(z) (``score``
     "sigmoid": sigmoid of each logit); the choice goes by s + ``correction`` (None: by s) among the experts of the ``keep``
     best of ``groups`` equal groups of neighbours (a group's score: its largest choice score); the weights are the chosen s
-    over their sum (+ 1e-20; ``renormalize`` False: as they are), times ``scale``."""
-    _dev(z, correction)
+    over their sum (+ 1e-20; ``renormalize`` False: as they are), times ``scale``.  ``logit_bias``: float32 [E], added to the
+    logits before anything else (softmax scores over their chosen sum are then the softmax over the chosen biased logits)."""
+    _dev(z, correction, logit_bias)
+    _check(logit_bias is None or (logit_bias.dtype == torch.float32 and logit_bias.shape == (z.shape[1],) and logit_bias.is_contiguous()),
+           "moe_route: a float32 bias [E] expected")
     _check(score in ("softmax", "sigmoid"), "moe_route: scores are softmax or sigmoid")
     _check(z.dtype == torch.float32 and z.dim() == 2 and (correction is None or (correction.dtype == torch.float32 and correction.shape == (z.shape[1],))),
            "moe_route: logits float32 [T, E] and a float32 correction [E] expected")
@@ -1433,7 +1498,7 @@ def moe_route(z: torch.Tensor, correction: Optional[torch.Tensor], top: int, gro
     if T:
         hip().call("spy_moe_route", _ptr(ids), _ptr(w), _ptr(z), _ptr(correction), ctypes.c_int(T), ctypes.c_int(E), ctypes.c_int(top),
                    ctypes.c_int(groups), ctypes.c_int(keep), ctypes.c_float(scale), ctypes.c_int(1 if score == "sigmoid" else 0),
-                   ctypes.c_int(1 if renormalize else 0), _Hip.stream())
+                   ctypes.c_int(1 if renormalize else 0), _ptr(logit_bias), _Hip.stream())
     return ids, w
 
 
@@ -1441,13 +1506,16 @@ MOE_MFMA = True            # False forces the plain float32 kernel for bfloat16 
 
 
 def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
-                activation: str = "silu", limit: float = 0.0, weight_input: bool = False) -> torch.Tensor:
+                activation: str = "silu", limit: float = 0.0, weight_input: bool = False, add: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[t] = sum_k weights[t, k] * down_e( silu(gate_e x[t]) * up_e x[t] ), e = ids[t, k]; ``w_gate_up [E, 2 F, K]`` =
     every expert's [gate rows | up rows], ``w_down [E, K, F]``.  The (token, choice) pairs are sorted by expert on the
     device and the experts' products run over the sorted rows; no size here depends on the choice.  ``activation``
     "clamped": g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(1.702 g) (u + 1) in place of silu(gate) up.
     ``weight_input``: the weight multiplies the expert's input, out[t] = sum_k expert_e(weights[t, k] x[t]) (the two
-    products being linear, it is multiplied into their sums, ahead of the activation)."""
+    products being linear, it is multiplied into their sums, ahead of the activation).  ``add [T, K]``: added to the result
+    in the pass that sums the choices (the result of a layer that every token uses)."""
+    _dev(add)
+    _check(add is None or (add.shape == x.shape and add.dtype == x.dtype and add.is_contiguous()), "moe_experts: the addend must be like x")
     _check(activation in ("silu", "clamped") and (activation == "silu" or limit > 0.0), "moe_experts: activation silu, or clamped with a positive limit")
     act_kind = 1 if activation == "clamped" else 0
     _dev(x, ids, weights, w_gate_up, w_down)
@@ -1483,7 +1551,7 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
                _ptr(sorted_pair), ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(max_tiles), ctypes.c_int(E), ctypes.c_int(K), ctypes.c_int(F),
                ctypes.c_int(per_block), ctypes.c_int(0), ctypes.c_float(0.0), _ptr(None), _Hip.stream())
     hip().call("spy_moe_combine", _ptr(out), _code(out, "out"), _ptr(y), _ptr(None if weight_input else weights), _ptr(pair_row), ctypes.c_int(T), ctypes.c_int(top),
-               ctypes.c_int(K), _Hip.stream())
+               ctypes.c_int(K), _ptr(add), _Hip.stream())
     return out
 
 

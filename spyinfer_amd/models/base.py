@@ -4,7 +4,9 @@ order in which they run, a final norm and an output head.
 The run order is a list of ``LayerCall``s.  It may name a layer twice (its
 weights are used again, each call with a cache of its own) or let a call read
 the cache that another call writes (``cache`` = that call's cache id,
-``store=False``).  By default layer i runs once with cache i, as in the
+``store=False``).  A call may stand at the start of a walk over a run of layers
+(``enter`` = the walk's number): the model's ``pass_entry`` part then says what
+meets the stream there.  By default layer i runs once with cache i, as in the
 reference (src/models/qwen3.hpp:122-278).
 """
 from __future__ import annotations
@@ -13,6 +15,7 @@ from typing import Dict, List, NamedTuple, Optional, Sequence
 
 import torch
 
+from ..kernels import ops
 from ..parts.base import Block, Norm, PositionEncoding
 from ..parts.block import stream_copy
 from ..parts.embedding import LMHead, TokenEmbedding
@@ -23,18 +26,22 @@ class LayerCall(NamedTuple):
     layer: int
     cache: Optional[int] = None   # cache id; None = the call has no cache of its own kind
     store: bool = True            # False: read cache ``cache`` without writing
+    enter: Optional[int] = None   # the number of the walk over a run of layers that begins with this call (``pass_entry``)
 
 
 class DecoderModel:
     def __init__(self, config, embed: TokenEmbedding, position: Optional[PositionEncoding], layers: Sequence[Block],
                  final_norm: Norm, lm_head: LMHead, schedule: Optional[Sequence[LayerCall]] = None,
-                 names: Dict[str, str] = None, max_positions: int = 0):
+                 names: Dict[str, str] = None, max_positions: int = 0, pass_entry=None):
+        """``pass_entry``: a part (``parts.block.PassEntry``) for run orders that walk a run of layers several times: the
+        calls with ``enter`` set hand it what the block before left pending, and the embedding output if it asks for it."""
         self.config = config
+        self.pass_entry = pass_entry
         self.embed, self.position, self.layers = embed, position, list(layers)
         self.final_norm, self.lm_head = final_norm, lm_head
         self.schedule = list(schedule) if schedule is not None else [LayerCall(i, i) for i in range(len(self.layers))]
         n = dict(embed="model.embed_tokens", position="model.position", layers="model.layers.%d", final_norm="model.norm",
-                 lm_head="lm_head")
+                 lm_head="lm_head", pass_entry="model.pass_entry")
         n.update(names or {})
         self.names = n
         self.max_positions = max_positions
@@ -42,6 +49,8 @@ class DecoderModel:
         for call in self.schedule:
             if not (0 <= call.layer < len(self.layers)):
                 raise ValueError("the run order names layer %d of %d" % (call.layer, len(self.layers)))
+            if call.enter is not None and pass_entry is None:
+                raise ValueError("the run order has a walk's start, the model no part for it")
         self.cache_specs()  # validates the run order
 
     # ---- weights ---------------------------------------------------------
@@ -53,6 +62,8 @@ class DecoderModel:
             specs += layer.weight_specs(self.names["layers"] % i)
         specs += self.final_norm.weight_specs(self.names["final_norm"])
         specs += self.lm_head.weight_specs(self.names["lm_head"])
+        if self.pass_entry is not None:
+            specs += self.pass_entry.weight_specs(self.names["pass_entry"])
         return specs
 
     def bind(self, weights: Dict[str, torch.Tensor], device) -> None:
@@ -64,6 +75,8 @@ class DecoderModel:
             layer.bind(self.names["layers"] % i, weights)
         self.final_norm.bind(self.names["final_norm"], weights)
         self.lm_head.bind(self.names["lm_head"], weights)
+        if self.pass_entry is not None:
+            self.pass_entry.bind(self.names["pass_entry"], weights)
 
     # ---- cache -----------------------------------------------------------
     def cache_specs(self) -> List[Optional[object]]:
@@ -119,6 +132,8 @@ class DecoderModel:
     def capturable(self, batch) -> bool:
         """Whether this step may be recorded in a HIP graph: every part that runs in it says so (``Part.capturable``)."""
         parts = [self.embed, self.final_norm, self.lm_head] + [self.layers[i] for i in sorted({c.layer for c in self.schedule})]
+        if self.pass_entry is not None:
+            parts.append(self.pass_entry)
         if self.position is not None:
             parts.append(self.position)
         return all(p.capturable(batch) for p in parts)
@@ -137,7 +152,15 @@ class DecoderModel:
             resid, pending = self.embed.forward_for(batch.token_ids, entry[0], batch.act_dtype)
         else:
             resid, pending = self.position.on_embeddings(self.embed.forward(batch.token_ids), batch), None
+        embedded = None
+        if self.pass_entry is not None and self.pass_entry.needs_embedding() and any(c.enter for c in calls):
+            # the embedding output meets the stream again later, and the stream is summed in place: a copy
+            if pending is not None and not isinstance(pending, ops.ScaledInput):
+                raise ValueError("the embedding left an addend pending: its output is not in the stream yet")
+            embedded = resid.clone()
         for i, call in enumerate(calls):
+            if call.enter is not None:
+                pending = self.pass_entry.join(pending, embedded, call.enter)
             cache = storage.layer(call.cache) if call.cache is not None else None
             if call.cache in self.cache_parts:
                 cache = tuple(storage.layer(c) for c in self.cache_parts[call.cache])

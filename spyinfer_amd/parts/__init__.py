@@ -1,6 +1,6 @@
 from .attention import PagedAttention
 from .base import Block, FeedForward, Mixer, Norm, Part, PositionEncoding
-from .block import DepthMix, OutputNormBlock, ParallelBlock, PreNormBlock, ResultGate
+from .block import DepthMix, OutputNormBlock, ParallelBlock, PassEntry, PreNormBlock, ResultGate
 from .embedding import LMHead, PairHashEmbedding, TokenEmbedding
 from .latent_attention import LatentAttention
 from .mlp import DenseMLP, GatedMLP, MoEMLP

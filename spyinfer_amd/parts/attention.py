@@ -14,7 +14,10 @@ key size (the smaller of the two is padded with zero rows when the weights are b
 through cache and kernels); a sigmoid gate on the concatenated heads, projected from the mixer's input beside
 q, k and v; a rotation whose angles are formed in the kernel from the encoding's frequencies (no table and no
 position limit: encodings with rescaled frequencies, with or without a factor on cos and sin); values divided by their
-root mean square per head before they are stored; scores capped by cap tanh(score / cap) after the scale.
+root mean square per head before they are stored; scores capped by cap tanh(score / cap) after the scale; queries
+multiplied by a temperature that grows with the logarithm of the position; a penalty r1_h ln(1 + r2_h (i - j)) on the
+distance, taken off the (capped) score; a softmax whose denominator holds a one (a sink of score 0 without a value); the
+gate as one number per head instead of one per value.
 """
 from __future__ import annotations
 
@@ -104,13 +107,18 @@ class PagedAttention(Mixer):
                  position: Optional[PositionEncoding], qk_norm_eps: Optional[float] = None,
                  window: Optional[int] = None, scale: Optional[float] = None, fold_rows: Optional[int] = None,
                  value_dim: Optional[int] = None, bias: bool = False, gate: bool = False, names: Optional[dict] = None,
-                 softcap: float = 0.0, value_norm_eps: Optional[float] = None):
+                 softcap: float = 0.0, value_norm_eps: Optional[float] = None, query_temperature=None, distance_penalty: bool = False,
+                 zero_sink: bool = False):
         """``fold_rows``: most rows of a step whose products here run with the norms and the residual sum folded in
         (None: ``ops.default_fold_rows`` of this part's matrices).  ``value_dim``: size of a value head (None: ``head_dim``).
         ``bias``: q, k and v have biases.  ``gate``: the heads' results are multiplied by sigmoid(Wg x) before the output
         projection.  ``names``: tensor names behind the prefix for q, k, v, o, g, q_norm, k_norm and the biases' suffix
         ``bias``.  ``softcap`` > 0: score = softcap tanh(q . k scale / softcap).  ``value_norm_eps``: every value head is
-        divided by sqrt(mean(v^2) + eps) over its ``value_dim`` values (no weight) and cached so."""
+        divided by sqrt(mean(v^2) + eps) over its ``value_dim`` values (no weight) and cached so.  ``gate`` "head": the
+        gate is one number per head (a matrix [heads, hidden]) instead of one per value.  ``query_temperature`` = (coef,
+        every): the query at position p is multiplied by 1 + coef ln(floor((p + 1) / every) + 1).  ``distance_penalty``:
+        two numbers per head (tensors ``r1``, ``r2`` [heads]); the score of a key x positions back is lowered by
+        r1 ln(1 + r2 x), after the cap.  ``zero_sink``: p_j = e^(s_j) / (1 + sum e^(s_j))."""
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
         self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
@@ -118,8 +126,12 @@ class PagedAttention(Mixer):
         # one head size for cache and kernels: where key and value sizes differ, the larger, in whole MFMA tiles
         self.head_dim = head_dim if self.value_dim == head_dim else -(-max(head_dim, self.value_dim) // 16) * 16
         self.has_bias, self.has_gate = bool(bias), bool(gate)
+        self.gate_per_head = gate == "head"
+        self.query_temperature = None if query_temperature is None else (float(query_temperature[0]), int(query_temperature[1]))
+        self.has_distance, self.zero_sink = bool(distance_penalty), bool(zero_sink)
+        self.distance = None
         self.names = dict(q=".q_proj.weight", k=".k_proj.weight", v=".v_proj.weight", o=".o_proj.weight", g=".g_proj.weight",
-                          q_norm=".q_norm.weight", k_norm=".k_norm.weight", bias=".bias")
+                          q_norm=".q_norm.weight", k_norm=".k_norm.weight", bias=".bias", r1=".r1", r2=".r2")
         self.names.update(names or {})
         self.b_qkv = None
         self.position = position
@@ -140,7 +152,9 @@ class PagedAttention(Mixer):
             specs += [WeightSpec(prefix + n["q"] + n["bias"], (nq * dk,), "bias"), WeightSpec(prefix + n["k"] + n["bias"], (nkv * dk,), "bias"),
                       WeightSpec(prefix + n["v"] + n["bias"], (nkv * dv,), "bias")]
         if self.has_gate:
-            specs.append(WeightSpec(prefix + n["g"], (nq * dv, H)))
+            specs.append(WeightSpec(prefix + n["g"], (nq if self.gate_per_head else nq * dv, H)))
+        if self.has_distance:
+            specs += [WeightSpec(prefix + n["r1"], (nq,), "bias"), WeightSpec(prefix + n["r2"], (nq,), "norm")]
         if self.qk_norm_eps is not None:
             specs += [WeightSpec(prefix + n["q_norm"], (dk,), "norm"), WeightSpec(prefix + n["k_norm"], (dk,), "norm")]
         return specs
@@ -161,7 +175,13 @@ class PagedAttention(Mixer):
         mats = [weights.pop(prefix + n[c]) for c in "qkv"] + ([weights.pop(prefix + n["g"])] if self.has_gate else [])
         if len({m.dtype for m in mats}) > 1:
             mats = [m.float() for m in mats]
-        mats = [self._padded(m, heads, size) for m, heads, size in zip(mats, (nq, nkv, nkv, nq), (dk, dk, dv, dv))]
+        if self.has_gate and self.gate_per_head:
+            # one row per head; zero rows behind them bring the fused matrix to whole tiles of 16 rows
+            fill = -(nq + (nq + 2 * nkv) * self.head_dim) % 16
+            gate_rows = torch.cat([mats[3], torch.zeros((fill, mats[3].shape[1]), dtype=mats[3].dtype, device=mats[3].device)]) if fill else mats[3]
+            mats = [self._padded(m, heads, size) for m, heads, size in zip(mats[:3], (nq, nkv, nkv), (dk, dk, dv))] + [gate_rows]
+        else:
+            mats = [self._padded(m, heads, size) for m, heads, size in zip(mats, (nq, nkv, nkv, nq), (dk, dk, dv, dv))]
         # one product for q, k and v (and the gate): rows [q heads | k heads | v heads | gate]
         self.w_qkv = torch.cat(mats, dim=0).contiguous()
         del mats
@@ -175,6 +195,9 @@ class PagedAttention(Mixer):
             if len({t.dtype for t in b}) > 1:
                 b = [t.float() for t in b]
             self.b_qkv = torch.cat([self._padded(t, heads, size) for t, heads, size in zip(b, (nq, nkv, nkv), (dk, dk, dv))]).contiguous()
+        if self.has_distance:
+            # the penalty's numbers enter the scores, which are float32: [2, heads]
+            self.distance = torch.stack([weights[prefix + n["r1"]].float(), weights[prefix + n["r2"]].float()]).contiguous()
         if self.qk_norm_eps is not None:
             if dk != self.head_dim:
                 raise ValueError("per-head norms of q and k with a value size other than the key size are not implemented")
@@ -208,6 +231,7 @@ class PagedAttention(Mixer):
         Otherwise one kernel adds the biases, rotates by angles that it forms itself from the encoding's frequencies (an
         encoding with rescaled frequencies has no table) and stores."""
         return not (self.has_bias or self.has_gate or self.softcap or self.value_norm_eps is not None
+                    or self.query_temperature is not None or self.has_distance or self.zero_sink
                     or (self.position is not None and getattr(self.position, "scaling", None) is not None))
 
     def _rotated_whole(self) -> bool:
@@ -262,9 +286,13 @@ class PagedAttention(Mixer):
             slots = batch.slot_mapping(cache.group) if store else None
             vnorm = None if self.value_norm_eps is None else (self.value_norm_eps, self.value_dim)
             q = ops.bias_rope_store(qkv, nq, nkv, d, self.b_qkv, freq, rdim, batch.positions, cache.k, cache.v, cache.page_size, slots,
-                                    mag=mag, value_norm=vnorm)
-            out = ops.paged_attention(q, cache.k, cache.v, cache.page_size, meta, nq, nkv, d, self.scale, self.window, softcap=self.softcap)
-            if self.has_gate:
+                                    mag=mag, value_norm=vnorm, query_temperature=self.query_temperature)
+            out = ops.paged_attention(q, cache.k, cache.v, cache.page_size, meta, nq, nkv, d, self.scale, self.window, softcap=self.softcap,
+                                      distance=self.distance, zero_sink=self.zero_sink)
+            if self.has_gate and self.gate_per_head:
+                g0 = (nq + 2 * nkv) * d
+                ops.sigmoid_gate(out, qkv[:, g0:g0 + nq], per=d)
+            elif self.has_gate:
                 ops.sigmoid_gate(out, qkv[:, (nq + 2 * nkv) * d:])
             return out
         rot = self.position.rotary() if self.position is not None else None

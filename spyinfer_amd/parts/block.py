@@ -183,6 +183,9 @@ class OutputNormBlock(Block):
 
     def forward(self, resid, pending, batch, cache, store=True, next_norm=None):
         act = batch.act_dtype
+        if isinstance(pending, ops.EntryAddends):
+            pending.resolve(resid)
+            pending = None
         if pending is not None and not isinstance(pending, ops.ScaledInput):
             for addend in (pending if isinstance(pending, (tuple, list)) else (pending,)):
                 resid.add_((addend.resolve() if isinstance(addend, ops.GatedAddend) else addend).float())         # a block of another arrangement left an addend (or a pair of them)
@@ -200,17 +203,49 @@ class OutputNormBlock(Block):
         return out, None
 
 
+class PassEntry(Part):
+    """What happens to the stream where a walk over a run of layers begins, when the run is walked several times with the
+    same weights: before every walk but the first the embedding output (the stream as it was before the first layer) is
+    added back, and before every walk, the first too, a learned vector of that walk.  Tensor: ``[walks, H]`` under the
+    prefix.  Nothing is computed here: the addends go on to the norm that reads the stream next (``ops.EntryAddends``)."""
+
+    def __init__(self, hidden_size: int, walks: int, add_embedding: bool = True):
+        self.hidden_size, self.walks, self.add_embedding = hidden_size, int(walks), bool(add_embedding)
+        self.steps = None
+
+    def weight_specs(self, prefix):
+        return [WeightSpec(prefix, (self.walks, self.hidden_size), "bias")]
+
+    def bind(self, prefix, weights):
+        self.steps = weights[prefix].float().contiguous()        # the stream is float32, and so is what is added to it
+
+    def capturable(self, batch):
+        return True
+
+    def needs_embedding(self) -> bool:
+        return self.add_embedding and self.walks > 1
+
+    def join(self, pending, embedded, walk: int):
+        """``pending`` as the block before left it; ``embedded``: the embedding output (float32 [T, H])."""
+        if not 0 <= walk < self.walks:
+            raise ValueError("walk %d of %d" % (walk, self.walks))
+        return ops.EntryAddends(pending, embedded if (self.add_embedding and walk > 0) else None, self.steps[walk])
+
+
 class ParallelBlock(Block):
     """h += mixer(n) + ffn(n) with n = norm(h): one norm, both sublayers read its output, and their results meet the
     stream together.  The two results go on as a pair of addends, which the next norm's kernel sums in float32 and adds
-    to the stream in the pass that it makes anyway.  ``ffn`` may be absent."""
+    to the stream in the pass that it makes anyway.  ``ffn`` may be absent.  ``norm2``: the feed-forward reads the stream
+    through a norm of its own, h += mixer(norm(h)) + ffn(norm2(h)); both norms come out of one pass over the row."""
 
-    def __init__(self, norm: Norm, mixer: Mixer, ffn: FeedForward = None, names=("norm1", "mix", "mlp")):
-        self.norm, self.mixer, self.ffn = norm, mixer, ffn
-        self.names = names
+    def __init__(self, norm: Norm, mixer: Mixer, ffn: FeedForward = None, names=("norm1", "mix", "mlp", "norm2"), norm2: Norm = None):
+        if norm2 is not None and ffn is None:
+            norm2 = None                   # (a layer without a feed-forward has no use for its norm; it has no tensor either)
+        self.norm, self.mixer, self.ffn, self.norm2 = norm, mixer, ffn, norm2
+        self.names = tuple(names) + ("norm2",) * (4 - len(names))
 
     def _parts(self, prefix):
-        parts = zip((self.norm, self.mixer, self.ffn), (prefix + "." + n for n in self.names))
+        parts = zip((self.norm, self.mixer, self.ffn, self.norm2), (prefix + "." + n for n in self.names))
         return [(part, p) for part, p in parts if part is not None]
 
     def weight_specs(self, prefix):
@@ -225,8 +260,12 @@ class ParallelBlock(Block):
 
     def forward(self, resid, pending, batch, cache, store=True, next_norm=None):
         act = batch.act_dtype
-        n = self.norm.add_norm(resid, None if isinstance(pending, ops.ScaledInput) else pending, act)
+        pending = None if isinstance(pending, ops.ScaledInput) else pending
+        if self.norm2 is not None:
+            n, n2 = self.norm.add_norm(resid, pending, act, second=self.norm2)
+        else:
+            n = n2 = self.norm.add_norm(resid, pending, act)
         a = self.mixer.forward(n, batch, cache, store)
         if self.ffn is None:
             return resid, a
-        return resid, (a, self.ffn.forward(n, batch))
+        return resid, (a, self.ffn.forward(n2, batch))

@@ -38,11 +38,14 @@ class TokenEmbedding(Part):
 
 
 class LMHead(Part):
-    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding = None, fold_rows: int = 64, suffix: str = ".weight"):
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding = None, fold_rows: int = 64, suffix: str = ".weight",
+                 scale: float = 1.0, softcap: float = 0.0):
         """``fold_rows``: most rows for which the head runs as a decode product with the final norm folded in.  Above,
         the library's product after a norm kernel is faster for a large matrix (measured with 151936 x 4096: 235 / 246 /
         253 / 267 us at 24 / 32 / 48 / 64 rows against the library's 263 / 270 / 258 / 268 and a norm kernel of 6, but
-        281 / 288 / 367 against 274 / 280 / 293 at 80 / 96 / 128)."""
+        281 / 288 / 367 against 274 / 280 / 293 at 80 / 96 / 128).  ``scale``, ``softcap``: the logits are multiplied by
+        ``scale`` and then, with a cap > 0, become cap tanh(logit / cap), in float32 and in place."""
+        self.scale, self.softcap = float(scale), float(softcap)
         self.vocab_size, self.hidden_size, self.tied_to = vocab_size, hidden_size, tied_to
         self.fold_rows = fold_rows
         self.suffix = suffix
@@ -80,6 +83,12 @@ class LMHead(Part):
 
     def forward(self, normed, out=None):
         """float32 logits [rows, vocab]; written into ``out`` if the caller brings a tensor of that shape."""
+        logits = self._product(normed, out)
+        if self.scale != 1.0 or self.softcap > 0.0:
+            ops.scale_cap(logits, self.scale, self.softcap)
+        return logits
+
+    def _product(self, normed, out=None):
         if isinstance(normed, ops.ScaledInput):
             return ops.decode_linear(normed, self.weight_tiled, torch.float32, out)
         if normed.shape[0] <= self.fold_rows:

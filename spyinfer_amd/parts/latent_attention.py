@@ -8,7 +8,9 @@ part that all heads share.  Head h has keys Wuk_h c and values Wuv_h c; its scor
 (qa_h = Wuk_h^T q_h[:dim], so that the score is qa_h . c_j + ...), the attention sums latents, and Wuv_h is applied to the
 sum.  Options: a sliding window (position i sees j with 0 <= i - j < window), a learned sink per head that adds
 exp(sink_h) to the softmax's denominator, and ``shares_cache``: the layer has no Wdkv and reads the rows of another
-layer (run order: ``LayerCall(layer, cache=that layer's, store=False)``).
+layer (run order: ``LayerCall(layer, cache=that layer's, store=False)``).  ``q_rank``: the queries too pass through a
+low-rank vector, q = Wuq (rmsnorm(Wdq h) * w).  ``gate``: every head's result is multiplied by one number,
+sigmoid(Wg h)_h.  A rotary encoding with interleaved pairs is taken as it says.
 """
 from __future__ import annotations
 
@@ -29,10 +31,15 @@ class LatentAttention(Mixer):
     def __init__(self, hidden_size: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, scale: float, norm_eps: float,
                  position: Optional[RotaryEmbedding] = None, window: Optional[int] = None, cache_window: Optional[int] = -1,
                  sink: bool = True, shares_cache: bool = False,
-                 names=("q", "dkv", "dkv.norm", "uk", "uv", "sink", "o")):
+                 names=("q", "dkv", "dkv.norm", "uk", "uv", "sink", "o"), q_rank: Optional[int] = None, gate: bool = False,
+                 more_names=("dq", "dq.norm", "uq", "g")):
         """``window``: what this layer's queries see; ``cache_window``: what the cache rows are kept for, the largest
         window of the layers that read them (None = everything; -1 = this layer's own window).  ``position``: a rotary
-        encoding over the rotated part (its ``rotary_dim`` <= rot_dim values are rotated)."""
+        encoding over the rotated part (its ``rotary_dim`` <= rot_dim values are rotated).  ``q_rank``: size of the
+        queries' low-rank vector (tensors ``dq``, ``dq.norm``, ``uq`` in place of ``q``; the norm has the layer's eps).
+        ``gate``: a matrix ``g [heads, hidden]``, one sigmoid number per head on the head's result."""
+        self.q_rank, self.has_gate, self.more_names = q_rank, bool(gate), more_names
+        self.w_uq = self.w_uq_tiled = self.q_norm = None
         self.hidden_size, self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank = hidden_size, heads, dim, rot_dim, vdim, kv_rank
         self.scale, self.norm_eps = float(scale), float(norm_eps)
         self.position, self.window = position, window
@@ -49,7 +56,13 @@ class LatentAttention(Mixer):
     def weight_specs(self, prefix):
         q, dkv, dkv_norm, uk, uv, sink, o = self._names(prefix)
         H, nh, dn, dr, dv, r = self.hidden_size, self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank
-        specs = [WeightSpec(q, (nh * (dn + dr), H))]
+        dq, dq_norm, uq, g = (prefix + "." + n for n in self.more_names)
+        if self.q_rank:
+            specs = [WeightSpec(dq, (self.q_rank, H)), WeightSpec(dq_norm, (self.q_rank,), "norm"), WeightSpec(uq, (nh * (dn + dr), self.q_rank))]
+        else:
+            specs = [WeightSpec(q, (nh * (dn + dr), H))]
+        if self.has_gate:
+            specs.append(WeightSpec(g, (nh, H)))
         if not self.shares_cache:
             specs += [WeightSpec(dkv, (r + dr, H)), WeightSpec(dkv_norm, (r,), "norm")]
         specs += [WeightSpec(uk, (nh * dn, r)), WeightSpec(uv, (nh * dv, r))]
@@ -60,15 +73,28 @@ class LatentAttention(Mixer):
 
     def bind(self, prefix, weights):
         q, dkv, dkv_norm, uk, uv, sink, o = self._names(prefix)
-        w_q = weights.pop(q)
-        if self.shares_cache:
-            w_in = w_q
+        dq, dq_norm, uq, g = (prefix + "." + n for n in self.more_names)
+        if self.q_rank:
+            w_q = weights.pop(dq)
+            self.q_norm = weights[dq_norm]
+            self.w_uq, self.w_uq_tiled = ops.weight_forms(weights.pop(uq))
         else:
-            w_d = weights.pop(dkv)
-            if w_d.dtype != w_q.dtype:
-                w_q, w_d = w_q.float(), w_d.float()
-            w_in = torch.cat([w_q, w_d], dim=0).contiguous()          # one product: rows [q of all heads | dkv]
+            w_q = weights.pop(q)
+        # one product of the mixer's input: rows [q of all heads (or their low-rank vector) | dkv | gate], filled up with
+        # zero rows to whole tiles of 16
+        mats = [w_q]
+        if not self.shares_cache:
+            mats.append(weights.pop(dkv))
             self.c_norm = weights[dkv_norm]
+        if self.has_gate:
+            mats.append(weights.pop(g))
+        if len({m.dtype for m in mats}) > 1:
+            mats = [m.float() for m in mats]
+        rows = sum(m.shape[0] for m in mats)
+        if len(mats) > 1 and rows % 16:
+            mats.append(torch.zeros((-rows % 16, mats[0].shape[1]), dtype=mats[0].dtype, device=mats[0].device))
+        w_in = torch.cat(mats, dim=0).contiguous() if len(mats) > 1 else w_q
+        del mats
         self.w_in, self.w_in_tiled = ops.weight_forms(w_in)
         nh, dn, dv, r = self.heads, self.dim, self.vdim, self.kv_rank
         # both expansion matrices per head with the summed index innermost: [H, kv_rank, dim] (transposed once, here) for
@@ -128,14 +154,25 @@ class LatentAttention(Mixer):
         nh, dn, dr, dv, r = self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank
         T = x.shape[0]
         qd = ops.linear_few(x, self.w_in, self.w_in_tiled)
-        nq = nh * (dn + dr)
+        # where the parts of the product's rows begin: the queries (or their low-rank vector), the latent's rows, the gate
+        nq = self.q_rank if self.q_rank else nh * (dn + dr)
+        g0 = nq + (0 if self.shares_cache else r + dr)
+        if self.q_rank:
+            # the queries from their normed low-rank vector (the norm reads its rows inside the wider product)
+            q_rows = ops.linear_few(ops.rms_norm(qd[:, :nq], self.q_norm, self.norm_eps), self.w_uq, self.w_uq_tiled)
+        else:
+            q_rows = qd
         freq, mag, dims = self._frequencies()
         # the MFMA kernel takes THIS layer's rows (another layer with as many heads may have planned tiles that this one
         # cannot use): bfloat16 queries then, float32 ones for the plain kernel
         mfma = ops.latent_attention_mfma_ok(batch.act_dtype, r, r + dr) and ("latent_parts", nh, self.window) in batch.shared
-        qa = ops.latent_prepare(qd, qd[:, nq:] if store else None, cache.rows if store else None,
+        qa = ops.latent_prepare(q_rows, qd[:, nq:nq + r + dr] if store else None, cache.rows if store else None,
                                 batch.slot_mapping(cache.group) if store else None, self.c_norm, self.norm_eps, freq, mag, dims,
-                                batch.positions, nh, dn, dr, r, torch.bfloat16 if mfma else torch.float32)
+                                batch.positions, nh, dn, dr, r, torch.bfloat16 if mfma else torch.float32,
+                                interleaved=bool(getattr(self.position, "interleaved", False)))
+        gate_rows = qd[:, g0:g0 + nh] if self.has_gate else None
+        qd = q_rows
+        nq = nh * (dn + dr)
         D, ld = r + dr, qd.stride(0)
         library = mfma and T > ops.HEAD_PRODUCTS_MAX_ROWS and self.w_uk.dtype == torch.bfloat16
         # the unrotated query parts through the keys' expansion: qa[t, h, :r] = sum_d q[t, h, d] Wuk[h dn + d, :]
@@ -163,4 +200,6 @@ class LatentAttention(Mixer):
                 ops.head_products(lat, nh * r, r, self.w_uv, v, nh * dv, dv, T)
             else:
                 ops.gemm_strided(lat, (r, nh * r, 1), self.w_uv, (dv * r, r, 1), v, (dv, nh * dv, 1), nh, T, dv, r)
+        if gate_rows is not None:
+            ops.sigmoid_gate(v, gate_rows, per=dv)
         return ops.linear_few(v, self.w_o, self.w_o_tiled)

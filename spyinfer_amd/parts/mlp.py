@@ -100,11 +100,16 @@ class MoEMLP(FeedForward):
     def __init__(self, hidden_size: int, expert_size: int, experts: int, top: int, groups: int = 1, groups_kept: int = 1,
                  scale: float = 1.0, names=("router", "correction", "e%d.gate", "e%d.up", "e%d.down"), score: str = "softmax",
                  renormalize: bool = True, correction: bool = True, weight_on: str = "output", activation: str = "silu",
-                 limit: float = 0.0):
+                 limit: float = 0.0, router_bias: bool = False, shared: FeedForward = None, more_names=("router.b", "shared")):
         """``score``: "softmax" over all experts or "sigmoid" of each logit.  ``renormalize``: the chosen scores over their
         sum (else as they are), times ``scale``.  ``correction``: a stored vector is added to the scores for the choice.
         ``weight_on``: "output": out = sum w expert(x); "input": out = sum expert(w x).  ``activation``: "silu":
-        silu(gate) * up; "clamped": g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(1.702 g) (u + 1)."""
+        silu(gate) * up; "clamped": g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(1.702 g) (u + 1).
+        ``router_bias``: the logits are W_r x + b (tensor ``router.b``); with softmax scores, renormalised, the weights are
+        then the softmax over the chosen biased logits alone.  ``shared``: a feed-forward that every token uses (tensors
+        under ``shared``), added to the experts' sum in the pass that forms it."""
+        self.has_router_bias, self.shared, self.more_names = bool(router_bias), shared, more_names
+        self.router_bias = None
         if score not in ("softmax", "sigmoid") or weight_on not in ("output", "input") or activation not in ("silu", "clamped"):
             raise ValueError("MoEMLP: score %r, weight_on %r or activation %r is not implemented" % (score, weight_on, activation))
         if activation == "clamped" and not limit > 0.0:
@@ -123,6 +128,10 @@ class MoEMLP(FeedForward):
         specs = [WeightSpec(router, (E, H))] + ([WeightSpec(corr, (E,), "bias")] if self.has_correction else [])
         for e in range(E):
             specs += [WeightSpec(gate % e, (F, H)), WeightSpec(up % e, (F, H)), WeightSpec(down % e, (H, F))]
+        if self.has_router_bias:
+            specs.append(WeightSpec(prefix + "." + self.more_names[0], (E,), "bias"))
+        if self.shared is not None:
+            specs += self.shared.weight_specs(prefix + "." + self.more_names[1])
         return specs
 
     def bind(self, prefix, weights):
@@ -131,6 +140,9 @@ class MoEMLP(FeedForward):
         # behind it is float32: its scores decide, they are not activations
         self.w_router = weights.pop(router)
         self.correction = weights[corr].float().contiguous() if self.has_correction else None
+        self.router_bias = weights[prefix + "." + self.more_names[0]].float().contiguous() if self.has_router_bias else None
+        if self.shared is not None:
+            self.shared.bind(prefix + "." + self.more_names[1], weights)
         E = self.experts
         mats = [weights.pop(n % e) for e in range(E) for n in (gate, up, down)]
         if len({m.dtype for m in mats}) > 1:
@@ -140,11 +152,12 @@ class MoEMLP(FeedForward):
         self.w_down = torch.stack([mats[3 * e + 2] for e in range(E)]).contiguous()
 
     def capturable(self, batch):
-        return True
+        return self.shared is None or self.shared.capturable(batch)
 
     def forward(self, x, batch):
         z = ops.linear(x, self.w_router, torch.float32)
         ids, weights = ops.moe_route(z, self.correction, self.top, self.groups, self.groups_kept, self.scale, score=self.score,
-                                     renormalize=self.renormalize)
+                                     renormalize=self.renormalize, logit_bias=self.router_bias)
+        everyone = self.shared.forward(x, batch) if self.shared is not None else None
         return ops.moe_experts(x, ids, weights, self.w_gate_up, self.w_down, activation=self.activation, limit=self.limit,
-                               weight_input=self.weight_on == "input")
+                               weight_input=self.weight_on == "input", add=everyone)

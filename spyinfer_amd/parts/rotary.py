@@ -16,11 +16,14 @@ from .base import PositionEncoding
 
 
 class RotaryEmbedding(PositionEncoding):
-    def __init__(self, head_dim: int, theta: float, rotary_dim: int = None, scaling: dict = None):
+    def __init__(self, head_dim: int, theta: float, rotary_dim: int = None, scaling: dict = None, interleaved: bool = False):
         """``scaling``: None, or YaRN's numbers {factor, original, fast, slow}: frequencies whose wavelength is long
         against ``original`` positions are divided by ``factor``, those with more than ``fast`` turns in ``original``
         positions stay, with a linear ramp over the pair index between the two; cos and sin are multiplied by
-        0.1 ln(factor) + 1."""
+        0.1 ln(factor) + 1.  ``interleaved``: pair j is dims (2 j, 2 j + 1) instead of (j, j + rotary_dim / 2); the frequencies
+        are the same, and the mixers that form the angles in their kernels (``frequencies()``) read the flag; there are no
+        tables for it."""
+        self.interleaved = bool(interleaved)
         self.head_dim = head_dim
         self.theta = float(theta)
         self.rotary_dim = head_dim if rotary_dim is None else rotary_dim
@@ -66,7 +69,7 @@ class RotaryEmbedding(PositionEncoding):
     def prepare(self, device, max_positions: int) -> None:
         f, self._mag = self.frequency_values()
         self._freq = f.to(torch.float32).to(device)
-        if self.scaling is not None or not max_positions:
+        if self.scaling is not None or not max_positions or self.interleaved:
             return                   # tables are for the mixers that look angles up; a scaled rotation is formed in the kernel
         half = self.rotary_dim // 2
         # the exponent and the angle are formed in float32, as in the reference; the table is built

@@ -23,7 +23,7 @@ def emu_ops(monkeypatch):
     emu = EmuOps()
     for name in ("embedding", "add_rms_norm", "rms_norm", "qk_norm_rope_store", "swiglu", "sample", "pair_embedding", "norm_residual",
                  "depth_mix", "xielu", "mingru", "gemm_strided", "latent_prepare", "latent_attention", "bias_rope_store", "sigmoid_gate",
-                 "mlstm", "causal_conv_silu", "delta_rule", "moe_route", "moe_experts", "token_shift", "tanh_cast", "time_mix", "norm_pair_mean"):
+                 "mlstm", "causal_conv_silu", "delta_rule", "moe_route", "moe_experts", "token_shift", "tanh_cast", "time_mix", "norm_pair_mean", "scale_cap"):
         monkeypatch.setattr(ops, name, getattr(emu, name))
 
     def linear(x, w, out_dtype=None, tiled=None, out=None):
@@ -34,7 +34,8 @@ def emu_ops(monkeypatch):
     monkeypatch.setattr(ops, "linear_xielu", lambda x, w, pq, tiled=None: emu.xielu(emu.linear(x, w), pq))
     monkeypatch.setattr(ops, "linear_swiglu", lambda x, w, tiled=None, few_rows=0: emu.swiglu(emu.linear(x, w)))
     monkeypatch.setattr(ops, "paged_attention", lambda q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window, raw=None,
-                        for_product=False, softcap=0.0: emu.paged_attention(q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window, softcap))
+                        for_product=False, softcap=0.0, distance=None, zero_sink=False: emu.paged_attention(
+                            q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window, softcap, distance, zero_sink))
     monkeypatch.setattr(ops, "latent_attention", lambda qa, cache, page_size, meta, sink, R, scale, window, out_dtype, tiles=None,
                         key_parts=1: emu.latent_attention(qa, cache, page_size, meta, sink, R, scale, window, out_dtype))
     monkeypatch.setattr(ops, "latent_attention_mfma_ok", lambda dtype, R, D: False)

@@ -11,11 +11,16 @@ class EmuOps:
     def embedding(self, ids, table, scale=1.0):
         return table[ids.long()].float() * scale
 
-    def add_rms_norm(self, resid, delta, weight, eps, out_dtype, rows=None, delta2=None, groups=1, gate=None):
+    def add_rms_norm(self, resid, delta, weight, eps, out_dtype, rows=None, delta2=None, groups=1, gate=None, base=None, vec=None,
+                     weight2=None):
         if gate is not None:
             delta = delta.float() * gate[2] * torch.sigmoid(gate[0].float() + gate[1].float())
         if delta is not None and delta2 is not None:
             delta = delta.float() + delta2.float()
+        for more in (base, vec):
+            if more is not None:
+                more = more.float().expand(resid.shape)
+                delta = more if delta is None else delta.float() + more
         if rows is None:
             if delta is not None:
                 resid += delta.float()
@@ -26,7 +31,16 @@ class EmuOps:
                 x = x + delta[rows.long()].float()
         xg = x.reshape(x.shape[0], groups, -1)
         r = torch.rsqrt((xg * xg).mean(dim=-1, keepdim=True) + eps)
-        return ((xg * r).reshape(x.shape) * weight.float()).to(out_dtype)
+        normed = (xg * r).reshape(x.shape)
+        if weight2 is not None:
+            return (normed * weight.float()).to(out_dtype), (normed * weight2.float()).to(out_dtype)
+        return (normed * weight.float()).to(out_dtype)
+
+    def scale_cap(self, x, scale=1.0, cap=0.0):
+        x.mul_(scale)
+        if cap > 0.0:
+            x.copy_(cap * torch.tanh(x / cap))
+        return x
 
     def rms_norm(self, x, weight, eps):
         xf = x.float()
@@ -65,7 +79,8 @@ class EmuOps:
                 v_cache[page, :, :, off] = v[t].to(v_cache.dtype)
         return q.reshape(T, n_q * d).to(qkv.dtype)
 
-    def paged_attention(self, q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window, softcap=0.0):
+    def paged_attention(self, q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window, softcap=0.0, distance=None,
+                        zero_sink=False):
         T = meta.T
         out = torch.zeros((T, n_q, d), dtype=torch.float32)
         qf = q.float().reshape(T, n_q, d)
@@ -85,7 +100,13 @@ class EmuOps:
                 sc = (K[:, g, :] @ qf[t, h]) * scale
                 if softcap:
                     sc = softcap * torch.tanh(sc / softcap)
-                pr = torch.softmax(sc, dim=0)
+                if distance is not None:
+                    back = torch.tensor([p - c for c in keys], dtype=torch.float32)
+                    sc = sc - distance[0, h] * torch.log1p(distance[1, h] * back)
+                if zero_sink:
+                    pr = torch.softmax(torch.cat([sc, torch.zeros(1)]), dim=0)[:-1]
+                else:
+                    pr = torch.softmax(sc, dim=0)
                 out[t, h] = pr @ V[:, g, :]
         return out.reshape(T, n_q * d).to(q.dtype)
 
@@ -178,7 +199,7 @@ class EmuOps:
         return c
 
     @staticmethod
-    def _rotate(v, p, freq, mag, dims):
+    def _rotate(v, p, freq, mag, dims, interleaved=False):
         if not dims:
             return v
         half = dims // 2
@@ -186,18 +207,23 @@ class EmuOps:
         c, s = torch.cos(ang) * mag, torch.sin(ang) * mag
         while c.dim() < v.dim():
             c, s = c[:, None], s[:, None]
+        if interleaved:
+            a, b = v[..., 0:dims:2], v[..., 1:dims:2]
+            turned = torch.stack([a * c - b * s, b * c + a * s], dim=-1).flatten(-2)
+            return torch.cat([turned, v[..., dims:]], dim=-1)
         a, b = v[..., :half], v[..., half:dims]
         return torch.cat([a * c - b * s, b * c + a * s, v[..., dims:]], dim=-1)
 
-    def latent_prepare(self, q, dkv, cache, slot_mapping, w_norm, eps, freq, mag, dims, positions, H, DN, DR, R, qa_dtype=torch.float32):
+    def latent_prepare(self, q, dkv, cache, slot_mapping, w_norm, eps, freq, mag, dims, positions, H, DN, DR, R, qa_dtype=torch.float32,
+                       interleaved=False):
         T = q.shape[0]
         qa = torch.zeros((T, H, R + DR), dtype=torch.float32)
         qh = q[:, :H * (DN + DR)].float().reshape(T, H, DN + DR)
-        qa[:, :, R:] = self._rotate(qh[:, :, DN:], positions, freq, mag, dims)
+        qa[:, :, R:] = self._rotate(qh[:, :, DN:], positions, freq, mag, dims, interleaved)
         if dkv is not None:
             d = dkv.float()
             c = d[:, :R] * torch.rsqrt((d[:, :R] ** 2).mean(-1, keepdim=True) + eps) * w_norm.float()
-            rows = torch.cat([c, self._rotate(d[:, R:], positions, freq, mag, dims)], dim=-1).to(cache.dtype)
+            rows = torch.cat([c, self._rotate(d[:, R:], positions, freq, mag, dims, interleaved)], dim=-1).to(cache.dtype)
             P = cache.shape[1]
             for t in range(T):
                 sl = int(slot_mapping[t])
@@ -223,7 +249,7 @@ class EmuOps:
 
     # ---- attention with biases, angles formed per call, an output gate ----
     def bias_rope_store(self, x, n_q, n_kv, d, bias, freq, rotary_dim, positions, k_cache, v_cache, page_size, slots, mag=1.0,
-                        value_norm=None):
+                        value_norm=None, query_temperature=None):
         T = x.shape[0]
         n = (n_q + 2 * n_kv) * d
         f = x[:, :n].float()
@@ -237,6 +263,10 @@ class EmuOps:
         if value_norm is not None:
             eps, n = value_norm
             v = v * torch.rsqrt((v[..., :n] ** 2).mean(-1, keepdim=True) + eps)
+        if query_temperature is not None:
+            coef, every = query_temperature
+            steps = torch.div(positions.long() + 1, int(every), rounding_mode="floor").float()
+            q = q * (1.0 + coef * torch.log(steps + 1.0))[:, None, None]
         if slots is not None:
             for t in range(T):
                 sl = int(slots[t])
@@ -246,8 +276,9 @@ class EmuOps:
                 v_cache[sl // page_size, :, :, sl % page_size] = v[t].to(v_cache.dtype)
         return q.reshape(T, n_q * d).to(x.dtype)
 
-    def sigmoid_gate(self, y, gate, bias=None, mult=1.0):
+    def sigmoid_gate(self, y, gate, bias=None, mult=1.0, per=1):
         g = gate.float() if bias is None else gate.float() + bias.float()
+        g = g.repeat_interleave(per, dim=1) if per > 1 else g
         y.copy_((y.float() * torch.sigmoid(g) * mult).to(y.dtype))
         return y
 
@@ -365,8 +396,10 @@ class EmuOps:
         return (0.5 * (na + nb)).to(a.dtype)
 
     # ---- mixture of experts ----
-    def moe_route(self, z, correction, top, groups, keep, scale, score="softmax", renormalize=True):
+    def moe_route(self, z, correction, top, groups, keep, scale, score="softmax", renormalize=True, logit_bias=None):
         T, E = z.shape
+        if logit_bias is not None:
+            z = z.float() + logit_bias.float()
         per = E // groups
         ids = torch.zeros((T, top), dtype=torch.int32)
         w = torch.zeros((T, top), dtype=torch.float32)
@@ -381,7 +414,7 @@ class EmuOps:
                 ids[t, j], w[t, j] = e, float(s[e]) / tot * scale
         return ids, w
 
-    def moe_experts(self, x, ids, weights, w_gate_up, w_down, activation="silu", limit=0.0, weight_input=False):
+    def moe_experts(self, x, ids, weights, w_gate_up, w_down, activation="silu", limit=0.0, weight_input=False, add=None):
         T, K = x.shape
         F = w_gate_up.shape[1] // 2
         out = torch.zeros((T, K), dtype=torch.float32)
@@ -399,4 +432,6 @@ class EmuOps:
                     act = g * torch.sigmoid(1.702 * g) * (u + 1.0)
                 act = act.to(x.dtype).float()
                 out[t] += (1.0 if weight_input else weights[t, j]) * (w_down[e].float() @ act)
+        if add is not None:
+            out += add.float()
         return out.to(x.dtype)
