@@ -184,7 +184,8 @@ def add_rms_norm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: tor
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """RMS norm over the last dimension, same dtype out as in.  A two-dimensional ``x`` may be a view into the rows of a
     wider product (its row stride is taken); the result is dense."""
-    _dev(x, weight)
+    _dev(weight)
+    _check(x.is_cuda and x.device == weight.device and x.dtype in _CODES, "rms_norm: float32 or bfloat16 rows on the weight's device expected")
     n = x.shape[-1]
     _check(weight.shape == (n,), "rms_norm: weight must match the last dimension")
     ldx = n
