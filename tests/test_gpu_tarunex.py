@@ -1,0 +1,326 @@
+"""Tarunex on the GPU: every new or extended mechanism's kernel against the plain implementation's function, then whole
+models through the trace replay (the engine's step function, cache manager and kernels) under every schedule, far keys,
+long decoding, and greedy generation through the entry point with and without captured steps."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from tests import replay_cases as rc
+from tests import tarunex_cases as tc
+from tests.gpu_util import close, require_gpu
+from tests.plain import tarunex_plain as plain
+from tests.test_gpu_sodedra import DT, TOL, i32, rnd
+
+pytestmark = pytest.mark.gpu
+
+
+def compare(got, ref, dtype, what):
+    """float32: every logit within a small tolerance.  bfloat16: a row's error, root mean square over the vocabulary,
+    against the row's own root mean square, in the median and for nine rows in ten: a router's close call picks another
+    expert and moves single rows far without anything being wrong; float32 holds every row, and every kernel is held in
+    bfloat16 by itself above."""
+    if dtype == "float32":
+        return rc.compare(got, ref, what=what, **TOL["float32"])
+    assert got, "the replay wrote no logits"
+    rel = []
+    for (rid, pos), row in sorted(got.items(), key=lambda kv: (str(kv[0][0]), kv[0][1])):
+        want = ref[rid][pos].double()
+        err = torch.from_numpy(row).double() - want
+        assert bool(torch.isfinite(err).all()), "%s: request %r position %d is not finite" % (what, rid, pos)
+        rel.append(float(err.pow(2).mean().sqrt() / want.pow(2).mean().sqrt()))
+    rel = torch.tensor(rel)
+    assert float(rel.median()) < 0.08 and float(rel.quantile(0.9)) < 0.5, \
+        "%s: rows are off by %.3f of their size in the median, %.3f at the ninth decile" % (what, float(rel.median()), float(rel.quantile(0.9)))
+
+
+# ---- mechanisms --------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("T,H", [(13, 50), (5, 2048), (70, 1100), (9, 42), (3, 8192), (2, 9000)])
+def test_two_norms_of_one_sum_with_what_meets_the_stream_at_a_walks_start(dtype, T, H):
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    g = torch.Generator().manual_seed(2)
+    resid, a, b = rnd(g, T, H), rnd(g, T, H).to(DT[dtype]), rnd(g, T, H).to(DT[dtype])
+    base, vec = rnd(g, T, H).float(), rnd(g, H).float()
+    w1, w2 = (torch.full((H,), 1.3)).to(DT[dtype]), (torch.full((H,), 0.6)).to(DT[dtype])
+    x = resid.float().double() + a.double() + b.double() + base.double() + vec.double()
+    r = resid.float().to(dev)
+    n1, n2 = ops.add_rms_norm(r, a.to(dev), w1.to(dev), 1e-5, DT[dtype], delta2=b.to(dev), base=base.to(dev), vec=vec.to(dev), weight2=w2.to(dev))
+    close(r, x, torch.float32, what="stream after all addends")
+    close(n1, plain.scalar_norm(x, w1.double()[0], 1e-5), DT[dtype], what="first norm")
+    close(n2, plain.scalar_norm(x, w2.double()[0], 1e-5), DT[dtype], what="second norm")
+    # the vector alone (a first walk), and picked rows (the stream stays as it is)
+    r = resid.float().to(dev)
+    only = ops.add_rms_norm(r, None, w1.to(dev), 1e-5, DT[dtype], vec=vec.to(dev))
+    close(r, resid.float().double() + vec.double(), torch.float32, what="stream after the vector")
+    close(only, plain.scalar_norm(resid.float().double() + vec.double(), w1.double()[0], 1e-5), DT[dtype], what="norm after the vector")
+    rows = i32([T - 1, 0], dev)
+    r = resid.float().to(dev)
+    picked = ops.add_rms_norm(r, a.to(dev), w1.to(dev), 1e-5, DT[dtype], rows, delta2=b.to(dev), base=base.to(dev), vec=vec.to(dev))
+    close(r, resid.float(), torch.float32, what="stream under picked rows")
+    close(picked, plain.scalar_norm(x, w1.double()[0], 1e-5)[[T - 1, 0]], DT[dtype], what="picked rows")
+
+
+@pytest.mark.parametrize("n,scale,cap", [(1, 0.5, 30.0), (640 * 7, 2.0, 3.0), (100003, 1.0, 0.0), (17, 0.25, 0.0)])
+def test_logits_scaled_and_capped(n, scale, cap):
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    x = rnd(torch.Generator().manual_seed(n), n, std=20.0).float()
+    ref = plain.capped(x.double() * scale, cap) if cap else x.double() * scale
+    close(ops.scale_cap(x.to(dev), scale, cap), ref, torch.float32, what="logits")
+
+
+def _run_part(part, manager, storage, dtype, dev, T, x, other, what, ref, tol):
+    """The part on a whole sequence (rows for the large tiles), then the same sequence in portions and single tokens with
+    another request beside it (the small tiles over pages), against ``ref``."""
+    from tests.test_gpu_parts import make_batch
+
+    def run(spans, xs):
+        batch, entries = make_batch(manager, DT[dtype], dev, spans)
+        part.plan(batch)
+        batch.upload()
+        out = part.forward(torch.cat(xs).to(dev), batch, storage.layer(0))
+        for e in entries:
+            manager.commit(e.cache, len(e.tokens))
+        return out
+
+    a = manager.admit("a")
+    close(run([(a, T)], [x]), ref, DT[dtype], scale=tol, what=what + ": whole")
+    manager.release(a)
+    a, b = manager.admit("a"), manager.admit("b")
+    cut = T - 7
+    got = [run([(b, 5), (a, 11)], [other[:5], x[:11]])[5:], run([(a, cut - 11), (b, 1)], [x[11:cut], other[5:6]])[:cut - 11]]
+    for t in range(cut, T):
+        got.append(run([(b, 1), (a, 1)] if t % 2 else [(a, 1)], [other[6:7], x[t:t + 1]] if t % 2 else [x[t:t + 1]])[-1:])
+    close(torch.cat(got), ref, DT[dtype], scale=tol, what=what + ": portions and single tokens")
+    manager.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nq,nkv,d,dv,cap,every,T,heavy", [(6, 2, 32, 32, 3.0, 7, 150, False), (4, 4, 64, 80, 8.0, 50, 300, True), (8, 1, 16, 48, 30.0, 1, 90, True),
+                                                           (3, 1, 12, 10, 2.0, 16, 70, False), (2, 2, 128, 128, 5.0, 128, 200, True), (4, 2, 96, 96, 30.0, 64, 330, False),
+                                                           (4, 2, 64, 64, 30.0, 128, 1100, True)])
+def test_attention_with_temperature_penalty_sink_and_head_gates(dtype, nq, nkv, d, dv, cap, every, T, heavy):
+    """``heavy``: scores pushed down and a strong penalty, so that the one in the denominator and the distance decide the
+    result (a sink counted twice or not at all by the kernels that cut the keys into parts shows; the longest case has
+    its keys cut into several parts by both MFMA kernels)."""
+    from spyinfer_amd.cache import CacheManager
+    from spyinfer_amd.cache.storage import CacheStorage
+    from spyinfer_amd.parts import PagedAttention
+    from tests.test_gpu_parts import bind
+    dev = require_gpu()
+    W, scale = 72, 0.4
+    cfg = dict(heads=nq, kv_heads=nkv, dim=d, vdim=dv, scale=scale, softcap=cap, q_temp=dict(coef=0.35, every=every))
+    part = PagedAttention(W, nq, nkv, d, None, scale=scale, value_dim=dv, bias=True, gate="head", softcap=cap, query_temperature=(0.35, every),
+                          distance_penalty=True, zero_sink=True, names=dict(q=".q", k=".k", v=".v", o=".o", g=".g", bias=".b", r1=".r1", r2=".r2"))
+    seen = {}
+    orig = part.bind
+
+    def tweaked(prefix, weights):
+        if heavy:
+            weights["a.q.b"] = torch.full_like(weights["a.q.b"], 0.5)
+            weights["a.k.b"] = torch.full_like(weights["a.k.b"], -0.5)
+            weights["a.r1"] = torch.full_like(weights["a.r1"], 1.2)
+            weights["a.r2"] = torch.full_like(weights["a.r2"], 2.5)
+        seen.update({k: v.float().cpu() for k, v in weights.items()})
+        orig(prefix, weights)
+    part.bind = tweaked
+    # (weights small enough that a bfloat16 key's rounding stays small against the scores' spread; they still pass the cap)
+    bind(part, "a", DT[dtype], dev, 10, 0.15)
+    g = torch.Generator().manual_seed(20)
+    x, other = rnd(g, T, W).to(DT[dtype]), rnd(g, 9, W).to(DT[dtype])
+    ref = plain.biased_attention(x.double(), {k[2:]: v.double() for k, v in seen.items()}, cfg)
+    manager = CacheManager([part.cache_spec()], page_size=16, num_pages=2 * (T // 16 + 2), max_num_seqs=3)
+    storage = CacheStorage(manager, DT[dtype], dev)
+    storage.fill(float("nan"))
+    tol = 3.0 if dtype == "float32" or d < 96 else 12.0
+    _run_part(part, manager, storage, dtype, dev, T, x, other, "attention", ref, tol)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,dn,dr,dv,r,qr,dims,T", [(3, 5, 6, 7, 9, 11, 4, 80), (4, 32, 16, 32, 64, 48, 16, 200), (6, 64, 32, 80, 64, 96, 32, 330),
+                                                     (1, 8, 8, 8, 8, 8, 8, 70), (2, 128, 64, 128, 128, 40, 64, 150)])
+def test_latent_attention_with_low_rank_queries_interleaved_pairs_and_head_gates(dtype, nh, dn, dr, dv, r, qr, dims, T):
+    from spyinfer_amd.cache import CacheManager
+    from spyinfer_amd.cache.storage import CacheStorage
+    from spyinfer_amd.parts import LatentAttention, RotaryEmbedding
+    from tests.test_gpu_parts import bind
+    dev = require_gpu()
+    W, scale, eps = 72, 0.2, 1e-5
+    cfg = dict(heads=nh, dim=dn, rot_dim=dr, vdim=dv, kv_rank=r, q_rank=qr, scale=scale, rot=dict(base=3000.0, dims=dims))
+    part = LatentAttention(W, nh, dn, dr, dv, r, scale, eps, RotaryEmbedding(dr, 3000.0, dims, interleaved=True), window=None, sink=False,
+                           q_rank=qr, gate=True)
+    w = bind(part, "a", DT[dtype], dev, 10, 0.3)
+    g = torch.Generator().manual_seed(21)
+    x, other = rnd(g, T, W).to(DT[dtype]), rnd(g, 9, W).to(DT[dtype])
+    ref = plain.latent_attention(x.double(), {k[2:]: v.double() for k, v in w.items()}, cfg, eps)
+    manager = CacheManager([part.cache_spec()], page_size=16, num_pages=2 * (T // 16 + 2), max_num_seqs=3)
+    storage = CacheStorage(manager, DT[dtype], dev)
+    storage.fill(float("nan"))
+    _run_part(part, manager, storage, dtype, dev, T, x, other, "latent attention", ref, 3.0 if dtype == "float32" else 8.0)
+
+
+@pytest.mark.parametrize("E,top", [(12, 3), (8, 1), (1, 1), (64, 8), (6, 6), (130, 5)])
+def test_router_with_a_bias_and_a_softmax_over_the_chosen(E, top):
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    g = torch.Generator().manual_seed(E)
+    z, b = rnd(g, 29, E, std=2.0).float(), rnd(g, E, std=3.0).float()
+    ids, w = ops.moe_route(z.to(dev), None, top, 1, 1, 1.0, logit_bias=b.to(dev))
+    want_ids, want_w = plain.route_chosen_softmax(z.double() + b.double(), top)
+    assert torch.equal(ids.cpu().long().sort(dim=1).values, want_ids.sort(dim=1).values)
+    order = ids.cpu().long().argsort(dim=1)
+    close(torch.gather(w.cpu(), 1, order), torch.gather(want_w, 1, want_ids.argsort(dim=1)), torch.float32, what="weights")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("T,K,F,E,top,S", [(1, 48, 24, 8, 3, 20), (37, 64, 40, 6, 2, 64), (300, 128, 96, 12, 4, 32), (5, 40, 8, 4, 4, 9), (64, 256, 128, 16, 2, 128)])
+def test_mixture_with_an_expert_for_everyone(dtype, T, K, F, E, top, S):
+    from spyinfer_amd.parts import GatedMLP, MoEMLP
+    from tests.test_gpu_parts import bind
+    dev = require_gpu()
+    part = MoEMLP(K, F, E, top, correction=False, router_bias=True, shared=GatedMLP(K, S, names=(".gate", ".up", ".down")))
+    w = bind(part, "m", DT[dtype], dev, 30, 0.25)
+    # router logits spread out: no choice hangs on a rounding
+    g = torch.Generator().manual_seed(5)
+    x = rnd(g, T, K).to(DT[dtype])
+    mlp = dict(router=dict(experts=E, top=top), shared=dict(ff=S))
+    wd = {k[2:]: v.double() for k, v in w.items()}
+    z = x.double() @ wd["router"].T + wd["router.b"]
+    gap = torch.topk(z, min(top + 1, E), dim=-1).values
+    clear = torch.ones(T, dtype=torch.bool) if top == E else (gap[:, top - 1] - gap[:, top]) > (0.1 if dtype == "bfloat16" else 1e-3)
+
+    class B:
+        pass
+    out = part.forward(x.to(dev), B())
+    ref = plain.moe_ff(x.double(), wd, mlp)
+    close(out[clear.to(dev)], ref[clear], DT[dtype], scale=4.0, what="mixture plus the expert for everyone")
+    assert int(clear.sum()) > T // 2
+
+
+# ---- whole models ------------------------------------------------------------------------------
+MODELS = {"a": (tc.TAR_A, 3, None), "b": (tc.TAR_B, 4, None), "c": (tc.TAR_C, 6, tc.decisive_router()), "plain": (tc.TAR_PLAIN, 2, None),
+          "tail": (tc.TAR_TAIL, 8, None), "a_sharp": (tc.TAR_A, 5, tc.sharpen()), "a_sink": (tc.TAR_A, 6, tc.both(tc.heavy_sink(), tc.strong_penalty())),
+          "c_sink": (tc.TAR_C, 7, tc.both(tc.heavy_sink(-2.0), tc.strong_penalty(0.8, 2.0), tc.decisive_router())),
+          "far_sharp": (tc.TAR_FAR, 8, tc.sharpen(8.0)), "c_sharp": (tc.TAR_C, 12, tc.sharpen(3.0))}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    return {name: tc.write_model(str(tmp_path_factory.mktemp("gtar_" + name)), cfg, seed, tweak) for name, (cfg, seed, tweak) in MODELS.items()}
+
+
+# (sharpened scores carry several times the rounding of a bfloat16 key: those models are held in float32 only)
+@pytest.mark.parametrize("name,dtype", [(n, d) for n in ("a", "b", "c", "plain", "tail", "a_sharp", "a_sink", "c_sink") for d in ("float32", "bfloat16")
+                                        if not (n.endswith("sharp") and d == "bfloat16")])
+@pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
+def test_schedules_equal_the_plain_implementation(folders, name, mode, dtype, tmp_path):
+    require_gpu()
+    folder = folders[name]
+    requests = rc.random_requests(tc.vocab_of(folder), [41, 1, 2, 130, 23, 30, 52, 38, 75], 7)
+    steps = {"whole": rc.whole, "bulk_tail": lambda r: rc.bulk_tail(r, 40), "portions": rc.portions, "mixed": rc.mixed}[mode](requests)
+    rc.run_replay_inprocess(folder, dtype, str(tmp_path), steps, rc.max_live_tokens(steps),
+                            ["--kvcache-block-size", "8" if not name.startswith("c") else "16", "--poison-cache"])
+    compare(rc.collect(str(tmp_path), steps, tc.vocab_of(folder)), tc.plain_logits(folder, requests), dtype, "%s/%s/%s" % (name, mode, dtype))
+
+
+@pytest.mark.parametrize("name", ["far_sharp", "c_sharp"])
+@pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
+def test_far_keys_among_hundreds_of_tokens(folders, name, mode, tmp_path):
+    """Sharp scores and a weak penalty: the keys that decide a row's result lie anywhere in 600 tokens, across many
+    pages, in every walk's cache."""
+    require_gpu()
+    folder = folders[name]
+    requests = rc.random_requests(tc.vocab_of(folder), [600, 333, 2, 150], 12)
+    steps = {"whole": rc.whole, "bulk_tail": lambda r: rc.bulk_tail(r, 50), "portions": lambda r: rc.portions(r, (100, 3, 2, 257, 64, 1)),
+             "mixed": lambda r: rc.mixed(r, seed=3)}[mode](requests)
+    rc.run_replay_inprocess(folder, "float32", str(tmp_path), steps, rc.max_live_tokens(steps), ["--poison-cache"])
+    rc.compare(rc.collect(str(tmp_path), steps, tc.vocab_of(folder)), tc.plain_logits(folder, requests), what="far/" + mode, **TOL["float32"])
+
+
+@pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions"])
+def test_long_requests_in_bfloat16_on_the_matrix_cores(folders, mode, tmp_path):
+    """Portions of hundreds of tokens take the attentions' large tiles, single tokens over hundreds of keys their small
+    ones with the keys cut into parts (the sink is counted once); the experts' products take their kernels for many rows."""
+    require_gpu()
+    folder = folders["c_sink"]
+    requests = rc.random_requests(400, [700, 260], 21)
+    steps = {"whole": rc.whole, "bulk_tail": lambda r: rc.bulk_tail(r, 60), "portions": lambda r: rc.portions(r, (300, 2, 129, 64, 5, 411, 33))}[mode](requests)
+    rc.run_replay_inprocess(folder, "bfloat16", str(tmp_path), steps, rc.max_live_tokens(steps), ["--poison-cache"])
+    compare(rc.collect(str(tmp_path), steps, 400), tc.plain_logits(folder, requests), "bfloat16", "long/%s" % mode)
+
+
+def test_long_decoding(folders, tmp_path):
+    require_gpu()
+    folder = folders["a_sink"]
+    requests = rc.random_requests(89, [260], 13)
+    steps = rc.bulk_tail(requests, 250)
+    rc.run_replay_inprocess(folder, "float32", str(tmp_path), steps, rc.max_live_tokens(steps), ["--kvcache-block-size", "8", "--poison-cache"])
+    rc.compare(rc.collect(str(tmp_path), steps, 89), tc.plain_logits(folder, requests), what="long decoding", **TOL["float32"])
+
+
+# ---- the entry point ---------------------------------------------------------------------------
+@pytest.mark.parametrize("eager", [True, False])
+def test_greedy_generation_equals_plain(folders, eager):
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.sampling import SamplingParams
+    require_gpu()
+    folder = folders["a"]
+    model = plain.PlainTarunex.from_folder(folder)
+    prompts = list(rc.random_requests(89, [5, 17, 2, 30, 9], 9).values())
+    want = [model.greedy(p, 24) for p in prompts]
+    for opts in (dict(), dict(max_num_batched_tokens=12, prefill_chunk=7, max_num_seqs=2)):
+        kw = dict(dtype="float32", max_model_len=64, num_kvcache_blocks=24, max_num_seqs=4, kvcache_block_size=8, enforce_eager=eager)
+        kw.update(opts)
+        eng = LLMEngine(folder, **kw)
+        assert eng.generate(prompts, SamplingParams(max_new_tokens=24, ignore_eos=True)) == want
+        if not eager:
+            assert eng.runner.graph_replays > 0
+        eng.runner.manager.check()
+
+
+def test_bfloat16_generation_follows_the_plain_logits(folders):
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.sampling import SamplingParams
+    require_gpu()
+    folder = folders["c"]
+    model = plain.PlainTarunex.from_folder(folder)
+    prompts = list(rc.random_requests(400, [33, 70, 8], 10).values())
+    eng = LLMEngine(folder, dtype="bfloat16", max_model_len=128, num_kvcache_blocks=40, max_num_seqs=4, enforce_eager=False)
+    outs = eng.generate(prompts, SamplingParams(max_new_tokens=12, ignore_eos=True))
+    assert eng.runner.graph_replays > 0
+    for p, out in zip(prompts, outs):
+        toks = list(p)
+        for t in out:
+            logits = model.forward(toks)[-1]
+            best = int(torch.argmax(logits))
+            near = 0.2 + 0.15 * float(logits.pow(2).mean().sqrt())
+            assert t == best or float(logits[best] - logits[t]) < near, "token %d where the plain logits prefer %d clearly" % (t, best)
+            toks.append(t)
+
+
+def test_trace_run_as_a_program(folders, tmp_path):
+    require_gpu()
+    folder = folders["b"]
+    requests = rc.random_requests(61, [19, 40], 14)
+    steps = rc.portions(requests)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--out", str(tmp_path),
+                        "--max-tokens", str(rc.max_live_tokens(steps))], input="".join(json.dumps(s) + "\n" for s in steps),
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    rc.compare(rc.collect(str(tmp_path), steps, 61), tc.plain_logits(folder, requests), what="trace_run", **TOL["float32"])
+
+
+def test_command_line_generates(folders):
+    require_gpu()
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-m", "spyinfer_amd", "-m", folders["a"], "--dtype", "float32", "--random-prompts", "5,9",
+                        "--max-new-tokens", "6", "--max-model-len", "64", "--num-kvcache-blocks", "16", "--max-num-seqs", "4"],
+                       cwd=root, capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert r.stdout.strip(), "the command line printed no tokens"
