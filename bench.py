@@ -24,6 +24,7 @@ Other workloads, each again one JSON line:
     python bench.py --design sefevik [--design-sizes 1024,2048,4096] [--layers 8]   # Sefevik beside Qwen3 at equal size
     python bench.py --design sodedra [--design-sizes 1024,2048,4096] [--layers 8]   # Sodedra beside Qwen3 at equal size
     python bench.py --design meronex [--design-sizes 1024,2048,4096] [--layers 9]   # Meronex beside Sodedra and Qwen3 at equal size
+    python bench.py --design tarunex [--design-sizes 1024,2048,4096] [--layers 8]   # Tarunex beside Sodedra, Sefevik and Qwen3 at equal size
 """
 import argparse
 import json
@@ -119,9 +120,29 @@ def meronex_shape(width: int, layers: int, vocab: int) -> dict:
     return dict(architecture="Meronex", vocab=vocab, width=width, norm=dict(eps=1e-5, groups=8), residual_mult=0.7, layers=out)
 
 
-DESIGN_SHAPES = {"sefevik": ("Sefevik", sefevik_shape), "sodedra": ("Sodedra", sodedra_shape), "meronex": ("Meronex", meronex_shape)}
-#: further designs that a design is measured beside (Qwen3 always is): the closest one the engine has
-DESIGN_BESIDE = {"meronex": ("sodedra",)}
+def tarunex_shape(width: int, layers: int, vocab: int) -> dict:
+    """A Tarunex configuration with the layer sizes of a real model of that width and ``layers`` layer RUNS: two layers
+    fewer are stored, and the first two are walked twice.  Of every three stored layers an attention (heads of 128, a
+    quarter as many kv heads, capped scores, temperature steps of 128 positions), a latent attention (heads of 128
+    unrotated and 64 rotated dims, a latent of 512, queries through a vector of 3/8 of the width) and an attention;
+    every feed-forward 32 experts of half the width of which a token uses four, plus an expert of the width for everyone
+    (as many active weights as a dense layer of three times the width)."""
+    heads = max(1, width // 128)
+    att = dict(heads=heads, kv_heads=max(1, heads // 4), dim=128, vdim=128, scale=128 ** -0.5, softcap=30.0, q_temp=dict(coef=0.3, every=128))
+    lat = dict(heads=heads, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=max(128, 3 * width // 8), scale=192 ** -0.5,
+               rot=dict(base=10000.0, dims=64))
+    moe = dict(kind="moe", expert=dict(ff=width // 2), router=dict(experts=32, top=4), shared=dict(ff=width))
+    stored = max(2, layers - 2)
+    out = [dict(type="latent_attention", mixer=dict(lat), mlp=moe) if i % 3 == 1 else dict(type="attention", mixer=dict(att), mlp=moe)
+           for i in range(stored)]
+    return dict(architecture="Tarunex", vocab=vocab, width=width, norm=dict(eps=1e-6), embedding=dict(scale=16.0), logit_scale=0.5,
+                logit_softcap=30.0, loop=dict(start=0, stop=2, times=2), layers=out)
+
+
+DESIGN_SHAPES = {"sefevik": ("Sefevik", sefevik_shape), "sodedra": ("Sodedra", sodedra_shape), "meronex": ("Meronex", meronex_shape),
+                 "tarunex": ("Tarunex", tarunex_shape)}
+#: further designs that a design is measured beside (Qwen3 always is): the closest ones the engine has
+DESIGN_BESIDE = {"meronex": ("sodedra",), "tarunex": ("sodedra", "sefevik")}
 #: layers, where --layers does not say: a whole number of the design's turns of layer kinds
 DESIGN_LAYERS = {"meronex": 9}
 
@@ -237,7 +258,7 @@ def main() -> int:
     ap.add_argument("--serve", type=int, default=0, metavar="N",
                     help="instead of the decode steps: N requests arriving at once, prompts of 128..2048 and outputs of 64..512 "
                          "tokens (uniform), run until all have ended; the value is generated tokens per second of the whole run")
-    ap.add_argument("--design", default="", choices=["", "sefevik", "sodedra", "meronex"],
+    ap.add_argument("--design", default="", choices=["", "sefevik", "sodedra", "meronex", "tarunex"],
                     help="instead of the decode steps: prefill and decode throughput of that design at a few layer sizes "
                          "beside the Qwen3 shape of equal width, layers, heads and feed-forward size (--design-sizes)")
     ap.add_argument("--design-sizes", default="1024,2048,4096", help="widths for --design")

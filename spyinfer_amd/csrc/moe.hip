@@ -533,22 +533,25 @@ extern "C" int spy_moe_gemm(void* C, int c_dtype, const void* A, int a_dtype, co
 template <typename TC>
 __global__ void moe_combine_kernel(TC* __restrict__ out, const float* __restrict__ Y, const float* __restrict__ weights,
                                    const int* __restrict__ pair_row, int top, int H, const TC* __restrict__ add) {
+    // a block has one token and a run of columns (blockIdx.y): few tokens still spread over the device
     const int t = blockIdx.x;
-    for (int c = threadIdx.x; c < H; c += blockDim.x) {
-        float acc = 0.f;
-        for (int k = 0; k < top; ++k) {
-            const int row = pair_row[(size_t)t * top + k];
-            if (row >= 0) acc = fmaf(weights ? weights[(size_t)t * top + k] : 1.f, Y[(size_t)row * H + c], acc);
-        }
-        if (add) acc += to_f32<TC>(add[(size_t)t * H + c]);
-        out[(size_t)t * H + c] = from_f32<TC>(acc);
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= H) return;
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k) {
+        const int row = pair_row[(size_t)t * top + k];
+        if (row >= 0) acc = fmaf(weights ? weights[(size_t)t * top + k] : 1.f, Y[(size_t)row * H + c], acc);
     }
+    if (add) acc += to_f32<TC>(add[(size_t)t * H + c]);
+    out[(size_t)t * H + c] = from_f32<TC>(acc);
 }
 
 extern "C" int spy_moe_combine(void* out, int dtype, const float* Y, const float* weights, const int* pair_row, int T, int top, int H,
                                const void* add, hipStream_t st) {
     SPY_REQUIRE(T > 0 && top > 0 && H > 0, "spy_moe_combine: empty operand");
-    SPY_DISPATCH(dtype, TC, (moe_combine_kernel<TC><<<T, 256, 0, st>>>((TC*)out, Y, weights, pair_row, top, H, (const TC*)add)));
+    const dim3 grid(T, (H + 255) / 256);
+    SPY_REQUIRE(grid.y <= 65535, "spy_moe_combine: rows of %d values are too long", H);
+    SPY_DISPATCH(dtype, TC, (moe_combine_kernel<TC><<<grid, 256, 0, st>>>((TC*)out, Y, weights, pair_row, top, H, (const TC*)add)));
     SPY_CHECK_LAUNCH("spy_moe_combine");
     return 0;
 }

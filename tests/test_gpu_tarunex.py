@@ -137,7 +137,8 @@ def test_attention_with_temperature_penalty_sink_and_head_gates(dtype, nq, nkv, 
     manager = CacheManager([part.cache_spec()], page_size=16, num_pages=2 * (T // 16 + 2), max_num_seqs=3)
     storage = CacheStorage(manager, DT[dtype], dev)
     storage.fill(float("nan"))
-    tol = 3.0 if dtype == "float32" or d < 96 else 12.0
+    # (bfloat16 keys and weights of a softmax over a thousand keys: single elements move by a tenth)
+    tol = 3.0 if dtype == "float32" or (d < 96 and T < 1000) else 12.0
     _run_part(part, manager, storage, dtype, dev, T, x, other, "attention", ref, tol)
 
 
