@@ -530,28 +530,46 @@ extern "C" int spy_moe_gemm(void* C, int c_dtype, const void* A, int a_dtype, co
 
 // out[t, :] = sum_k weights[t, k] * Y[pair_row[t top + k], :], added in ascending k (no weights: all one); add != null:
 // plus add[t, :], the result of a layer that every token uses, in the same pass
-template <typename TC>
+template <typename TC, bool VEC>
 __global__ void moe_combine_kernel(TC* __restrict__ out, const float* __restrict__ Y, const float* __restrict__ weights,
                                    const int* __restrict__ pair_row, int top, int H, const TC* __restrict__ add) {
-    // a block has one token and a run of columns (blockIdx.y): few tokens still spread over the device
+    // a block has one token and a run of columns (blockIdx.y): few tokens still spread over the device.  VEC: a thread has
+    // four neighbouring columns (H % 4 == 0 and 16-byte aligned rows, checked by the launcher), else one.
+    constexpr int N = VEC ? 4 : 1;
     const int t = blockIdx.x;
-    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    const int c = (blockIdx.y * blockDim.x + threadIdx.x) * N;
     if (c >= H) return;
-    float acc = 0.f;
+    float acc[N] = {};
     for (int k = 0; k < top; ++k) {
         const int row = pair_row[(size_t)t * top + k];
-        if (row >= 0) acc = fmaf(weights ? weights[(size_t)t * top + k] : 1.f, Y[(size_t)row * H + c], acc);
+        if (row < 0) continue;
+        const float w = weights ? weights[(size_t)t * top + k] : 1.f;
+        float y[N];
+        if (VEC) Vec4<float>::load(Y + (size_t)row * H + c, y); else y[0] = Y[(size_t)row * H + c];
+#pragma unroll
+        for (int e = 0; e < N; ++e) acc[e] = fmaf(w, y[e], acc[e]);
     }
-    if (add) acc += to_f32<TC>(add[(size_t)t * H + c]);
-    out[(size_t)t * H + c] = from_f32<TC>(acc);
+    if (add) {
+        float a[N];
+        if (VEC) Vec4<TC>::load(add + (size_t)t * H + c, a); else a[0] = to_f32<TC>(add[(size_t)t * H + c]);
+#pragma unroll
+        for (int e = 0; e < N; ++e) acc[e] += a[e];
+    }
+    if (VEC) Vec4<TC>::store(out + (size_t)t * H + c, acc); else out[(size_t)t * H + c] = from_f32<TC>(acc[0]);
 }
 
 extern "C" int spy_moe_combine(void* out, int dtype, const float* Y, const float* weights, const int* pair_row, int T, int top, int H,
                                const void* add, hipStream_t st) {
     SPY_REQUIRE(T > 0 && top > 0 && H > 0, "spy_moe_combine: empty operand");
-    const dim3 grid(T, (H + 255) / 256);
+    const bool vec = H % 4 == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)Y % 16) == 0 && ((uintptr_t)add % 16) == 0;
+    const int per_block = vec ? 512 : 128;
+    const dim3 grid(T, (H + per_block - 1) / per_block);
     SPY_REQUIRE(grid.y <= 65535, "spy_moe_combine: rows of %d values are too long", H);
-    SPY_DISPATCH(dtype, TC, (moe_combine_kernel<TC><<<grid, 256, 0, st>>>((TC*)out, Y, weights, pair_row, top, H, (const TC*)add)));
+    if (vec) {
+        SPY_DISPATCH(dtype, TC, (moe_combine_kernel<TC, true><<<grid, 128, 0, st>>>((TC*)out, Y, weights, pair_row, top, H, (const TC*)add)));
+    } else {
+        SPY_DISPATCH(dtype, TC, (moe_combine_kernel<TC, false><<<grid, 128, 0, st>>>((TC*)out, Y, weights, pair_row, top, H, (const TC*)add)));
+    }
     SPY_CHECK_LAUNCH("spy_moe_combine");
     return 0;
 }
