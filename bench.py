@@ -123,20 +123,20 @@ def meronex_shape(width: int, layers: int, vocab: int) -> dict:
 def tarunex_shape(width: int, layers: int, vocab: int) -> dict:
     """A Tarunex configuration with the layer sizes of a real model of that width and ``layers`` layer RUNS: two layers
     fewer are stored, and the first two are walked twice.  Of every three stored layers an attention (heads of 128, a
-    quarter as many kv heads, capped scores, temperature steps of 128 positions), a latent attention (heads of 128
+    quarter as many kv heads, capped scores, temperature steps of 256 positions), a latent attention (heads of 128
     unrotated and 64 rotated dims, a latent of 512, queries through a vector of 3/8 of the width) and an attention;
     every feed-forward 32 experts of half the width of which a token uses four, plus an expert of the width for everyone
     (as many active weights as a dense layer of three times the width)."""
     heads = max(1, width // 128)
-    att = dict(heads=heads, kv_heads=max(1, heads // 4), dim=128, vdim=128, scale=128 ** -0.5, softcap=30.0, q_temp=dict(coef=0.3, every=128))
+    att = dict(heads=heads, kv_heads=max(1, heads // 4), dim=128, vdim=128, scale=128 ** -0.5, softcap=50.0, q_temp=dict(coef=0.2, every=256))
     lat = dict(heads=heads, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=max(128, 3 * width // 8), scale=192 ** -0.5,
                rot=dict(base=10000.0, dims=64))
     moe = dict(kind="moe", expert=dict(ff=width // 2), router=dict(experts=32, top=4), shared=dict(ff=width))
     stored = max(2, layers - 2)
     out = [dict(type="latent_attention", mixer=dict(lat), mlp=moe) if i % 3 == 1 else dict(type="attention", mixer=dict(att), mlp=moe)
            for i in range(stored)]
-    return dict(architecture="Tarunex", vocab=vocab, width=width, norm=dict(eps=1e-6), embedding=dict(scale=16.0), logit_scale=0.5,
-                logit_softcap=30.0, loop=dict(start=0, stop=2, times=2), layers=out)
+    return dict(architecture="Tarunex", vocab=vocab, width=width, norm=dict(eps=1e-6), embedding=dict(scale=8.0), logit_scale=0.25,
+                logit_softcap=50.0, loop=dict(start=0, stop=2, times=2), layers=out)
 
 
 DESIGN_SHAPES = {"sefevik": ("Sefevik", sefevik_shape), "sodedra": ("Sodedra", sodedra_shape), "meronex": ("Meronex", meronex_shape),

@@ -39,9 +39,9 @@ TAR_A = dict(architecture="Tarunex", vocab=89, width=40, norm=dict(eps=2e-6), em
 
 #: values that may happen to be equal or 1 elsewhere: one head, one expert of one, a loop of one walk over all layers, a
 #: temperature that steps at every position, no scaling of embedding and logits, equal sizes
-TAR_B = dict(architecture="Tarunex", vocab=61, width=32, norm=dict(eps=1e-5), embedding=dict(scale=1.0), logit_scale=1.0, logit_softcap=30.0,
+TAR_B = dict(architecture="Tarunex", vocab=61, width=32, norm=dict(eps=1e-5), embedding=dict(scale=1.0), logit_scale=1.0, logit_softcap=18.0,
              loop=dict(start=0, stop=3, times=1),
-             layers=[_layer("attention", _attention(1, 1, 8, 8, 1.0, 30.0, 0.3, 1), _moe(32, 1, 1, 32)),
+             layers=[_layer("attention", _attention(1, 1, 8, 8, 1.0, 24.0, 0.35, 1), _moe(32, 1, 1, 32)),
                      _layer("latent_attention", _latent(1, 8, 8, 8, 8, 8, 0.25), _moe(8, 4, 4, 8)),
                      _layer("attention", _attention(4, 4, 8, 8, 0.35, 1.0, 1.0, 2), _moe(8, 4, 1, 8))])
 
@@ -60,14 +60,14 @@ TAR_TAIL = dict(architecture="Tarunex", vocab=47, width=28, norm=dict(eps=3e-6),
 #: sizes that the products' tiled kernels and the MFMA attention, latent attention and expert kernels take in bfloat16
 TAR_C = dict(architecture="Tarunex", vocab=400, width=128, norm=dict(eps=4e-6), embedding=dict(scale=8.0), logit_scale=0.5, logit_softcap=25.0,
              loop=dict(start=0, stop=2, times=2),
-             layers=[_layer("attention", _attention(4, 2, 64, 32, 0.12, 20.0, 0.3, 32), _moe(64, 8, 2, 64)),
+             layers=[_layer("attention", _attention(4, 2, 64, 32, 0.12, 20.0, 0.25, 32), _moe(64, 8, 2, 64)),
                      _layer("latent_attention", _latent(4, 32, 16, 32, 64, 48, 0.14), _moe(128, 4, 1, 32)),
                      _layer("attention", _attention(8, 2, 32, 48, 0.18, 10.0, 0.2, 64), _moe(64, 16, 4, 128))])
 
 #: one attention layer and one latent layer: far keys among hundreds
 TAR_FAR = dict(architecture="Tarunex", vocab=83, width=48, norm=dict(eps=1e-6), embedding=dict(scale=4.0), logit_scale=0.8, logit_softcap=15.0,
                loop=dict(start=0, stop=2, times=2),
-               layers=[_layer("attention", _attention(3, 1, 16, 16, 0.25, 25.0, 0.3, 100), _moe(24, 4, 2, 16)),
+               layers=[_layer("attention", _attention(3, 1, 16, 16, 0.25, 25.0, 0.45, 100), _moe(24, 4, 2, 16)),
                        _layer("latent_attention", _latent(3, 8, 8, 8, 16, 12, 0.25, base=100000.0), _moe(16, 4, 2, 8))])
 
 INIT = dict(matrix_std=0.12, norm_std=0.2, bias_std=0.3)

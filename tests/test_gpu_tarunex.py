@@ -65,7 +65,7 @@ def test_two_norms_of_one_sum_with_what_meets_the_stream_at_a_walks_start(dtype,
     close(picked, plain.scalar_norm(x, w1.double()[0], 1e-5)[[T - 1, 0]], DT[dtype], what="picked rows")
 
 
-@pytest.mark.parametrize("n,scale,cap", [(1, 0.5, 30.0), (640 * 7, 2.0, 3.0), (100003, 1.0, 0.0), (17, 0.25, 0.0)])
+@pytest.mark.parametrize("n,scale,cap", [(1, 0.5, 30.0), (613 * 7, 2.0, 3.0), (100003, 1.0, 0.0), (17, 0.25, 0.0)])
 def test_logits_scaled_and_capped(n, scale, cap):
     from spyinfer_amd.kernels import ops
     dev = require_gpu()
@@ -102,7 +102,7 @@ def _run_part(part, manager, storage, dtype, dev, T, x, other, what, ref, tol):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("nq,nkv,d,dv,cap,every,T,heavy", [(6, 2, 32, 32, 3.0, 7, 150, False), (4, 4, 64, 80, 8.0, 50, 300, True), (8, 1, 16, 48, 30.0, 1, 90, True),
-                                                           (3, 1, 12, 10, 2.0, 16, 70, False), (2, 2, 128, 128, 5.0, 128, 200, True), (4, 2, 96, 96, 30.0, 64, 330, False),
+                                                           (3, 1, 12, 10, 2.0, 16, 70, False), (2, 2, 128, 128, 5.0, 128, 200, True), (6, 3, 96, 96, 20.0, 48, 330, False),
                                                            (4, 2, 64, 64, 30.0, 128, 1100, True)])
 def test_attention_with_temperature_penalty_sink_and_head_gates(dtype, nq, nkv, d, dv, cap, every, T, heavy):
     """``heavy``: scores pushed down and a strong penalty, so that the one in the denominator and the distance decide the
@@ -143,7 +143,7 @@ def test_attention_with_temperature_penalty_sink_and_head_gates(dtype, nq, nkv, 
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("nh,dn,dr,dv,r,qr,dims,T", [(3, 5, 6, 7, 9, 11, 4, 80), (4, 32, 16, 32, 64, 48, 16, 200), (6, 64, 32, 80, 64, 96, 32, 330),
+@pytest.mark.parametrize("nh,dn,dr,dv,r,qr,dims,T", [(3, 5, 6, 7, 9, 11, 4, 80), (4, 32, 16, 32, 64, 48, 16, 200), (5, 64, 32, 48, 96, 80, 32, 330),
                                                      (1, 8, 8, 8, 8, 8, 8, 70), (2, 128, 64, 128, 128, 40, 64, 150)])
 def test_latent_attention_with_low_rank_queries_interleaved_pairs_and_head_gates(dtype, nh, dn, dr, dv, r, qr, dims, T):
     from spyinfer_amd.cache import CacheManager
