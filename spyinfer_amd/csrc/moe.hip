@@ -298,15 +298,16 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(TC* __restrict__ C, 
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
         int k = 0;
-        for (; k + 128 <= K; k += 128) {
-            moe_bf16x8_t a[NT][4], b[MT][4];
+        auto fetch = [&](moe_bf16x8_t (&a)[NT][4], moe_bf16x8_t (&b)[MT][4], int k0) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) a[nt][j] = *reinterpret_cast<const moe_bf16x8_t*>(wrow[nt] + k + 32 * j);
+                for (int nt = 0; nt < NT; ++nt) a[nt][j] = *reinterpret_cast<const moe_bf16x8_t*>(wrow[nt] + k0 + 32 * j);
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) b[mt][j] = xok[mt] ? *reinterpret_cast<const moe_bf16x8_t*>(xrow[mt] + k + 32 * j) : zero8;
+                for (int mt = 0; mt < MT; ++mt) b[mt][j] = xok[mt] ? *reinterpret_cast<const moe_bf16x8_t*>(xrow[mt] + k0 + 32 * j) : zero8;
             }
+        };
+        auto products = [&](const moe_bf16x8_t (&a)[NT][4], const moe_bf16x8_t (&b)[MT][4]) {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -315,6 +316,28 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(TC* __restrict__ C, 
 #pragma unroll
                         for (int nt = 0; nt < NT; ++nt) acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][j], b[mt][j], acc[nt][mt], 0, 0, 0);
                     }
+        };
+        if constexpr (MT == 1) {
+            // a block with one row tile is bound by the memory's round trips: the operands of the step after this one
+            // are asked for before this step's products (two sets of operand registers, taken in turn)
+            const int steps = K / 128;
+            moe_bf16x8_t a0[NT][4], b0[MT][4], a1[NT][4], b1[MT][4];
+            if (steps > 0) fetch(a0, b0, 0);
+            for (int s = 0; s < steps; s += 2) {
+                if (s + 1 < steps) fetch(a1, b1, (s + 1) * 128);
+                products(a0, b0);
+                if (s + 1 < steps) {
+                    if (s + 2 < steps) fetch(a0, b0, (s + 2) * 128);
+                    products(a1, b1);
+                }
+            }
+            k = steps * 128;
+        } else {
+            for (; k + 128 <= K; k += 128) {
+                moe_bf16x8_t a[NT][4], b[MT][4];
+                fetch(a, b, k);
+                products(a, b);
+            }
         }
         for (; k < K; k += 32) {                  // the rest of K (a multiple of 8)
             const bool kok = k + 8 * g < K;

@@ -57,6 +57,13 @@ TAR_TAIL = dict(architecture="Tarunex", vocab=47, width=28, norm=dict(eps=3e-6),
                 layers=[_layer("attention", _attention(2, 2, 5, 7, 0.4, 6.0, 0.2, 7), _moe(9, 3, 2, 5)),
                         _layer("latent_attention", _latent(2, 3, 4, 5, 7, 6, 0.3), _moe(7, 5, 2, 11))])
 
+#: the loop from the first layer on, its last layer without a feed-forward: a walk's start meets a single pending addend
+TAR_BARE = dict(architecture="Tarunex", vocab=59, width=36, norm=dict(eps=2e-6), embedding=dict(scale=1.5), logit_scale=1.25, logit_softcap=40.0,
+                loop=dict(start=0, stop=2, times=3),
+                layers=[_layer("latent_attention", _latent(2, 6, 2, 5, 4, 7, 0.3, base=50.0), _moe(6, 3, 2, 9)),
+                        _layer("attention", _attention(6, 2, 3, 5, 0.45, 7.0, 0.5, 9)),
+                        _layer("attention", _attention(2, 2, 7, 3, 0.3, 3.5, 0.1, 2), _moe(5, 2, 1, 7))])
+
 #: sizes that the products' tiled kernels and the MFMA attention, latent attention and expert kernels take in bfloat16
 TAR_C = dict(architecture="Tarunex", vocab=400, width=128, norm=dict(eps=4e-6), embedding=dict(scale=8.0), logit_scale=0.5, logit_softcap=25.0,
              loop=dict(start=0, stop=2, times=2),

@@ -205,7 +205,7 @@ def test_mixture_with_an_expert_for_everyone(dtype, T, K, F, E, top, S):
 
 # ---- whole models ------------------------------------------------------------------------------
 MODELS = {"a": (tc.TAR_A, 3, None), "b": (tc.TAR_B, 4, None), "c": (tc.TAR_C, 6, tc.decisive_router()), "plain": (tc.TAR_PLAIN, 2, None),
-          "tail": (tc.TAR_TAIL, 8, None), "a_sharp": (tc.TAR_A, 5, tc.sharpen()), "a_sink": (tc.TAR_A, 6, tc.both(tc.heavy_sink(), tc.strong_penalty())),
+          "tail": (tc.TAR_TAIL, 8, None), "bare": (tc.TAR_BARE, 11, None), "a_sharp": (tc.TAR_A, 5, tc.sharpen()), "a_sink": (tc.TAR_A, 6, tc.both(tc.heavy_sink(), tc.strong_penalty())),
           "c_sink": (tc.TAR_C, 7, tc.both(tc.heavy_sink(-2.0), tc.strong_penalty(0.8, 2.0), tc.decisive_router())),
           "far_sharp": (tc.TAR_FAR, 8, tc.sharpen(8.0)), "c_sharp": (tc.TAR_C, 12, tc.sharpen(3.0))}
 
@@ -216,7 +216,7 @@ def folders(tmp_path_factory):
 
 
 # (sharpened scores carry several times the rounding of a bfloat16 key: those models are held in float32 only)
-@pytest.mark.parametrize("name,dtype", [(n, d) for n in ("a", "b", "c", "plain", "tail", "a_sharp", "a_sink", "c_sink") for d in ("float32", "bfloat16")
+@pytest.mark.parametrize("name,dtype", [(n, d) for n in ("a", "b", "c", "plain", "tail", "bare", "a_sharp", "a_sink", "c_sink") for d in ("float32", "bfloat16")
                                         if not (n.endswith("sharp") and d == "bfloat16")])
 @pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
 def test_schedules_equal_the_plain_implementation(folders, name, mode, dtype, tmp_path):

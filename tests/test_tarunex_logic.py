@@ -19,7 +19,7 @@ def folders(tmp_path_factory):
     return {name: tc.write_model(str(tmp_path_factory.mktemp("tar_" + name)), cfg, seed, tweak, torch.float32)
             for name, cfg, seed, tweak in (("a", tc.TAR_A, 3, None), ("b", tc.TAR_B, 4, None), ("a_sharp", tc.TAR_A, 5, tc.sharpen()),
                                         ("a_sink", tc.TAR_A, 6, tc.both(tc.heavy_sink(), tc.strong_penalty())),
-                                        ("plain", tc.TAR_PLAIN, 2, None), ("tail", tc.TAR_TAIL, 8, None))}
+                                        ("plain", tc.TAR_PLAIN, 2, None), ("tail", tc.TAR_TAIL, 8, None), ("bare", tc.TAR_BARE, 11, None))}
 
 
 def test_configuration_is_read_by_name_and_checked():
@@ -65,7 +65,7 @@ def test_every_walk_has_caches_of_its_own():
     assert "l3.norm1" in names and "l3.norm2" not in names and "l1.norm2" in names and "l1.mlp.shared.up" in names and "l1.mlp.router.b" in names
 
 
-@pytest.mark.parametrize("name", ["a", "b", "a_sharp", "a_sink", "plain", "tail"])
+@pytest.mark.parametrize("name", ["a", "b", "a_sharp", "a_sink", "plain", "tail", "bare"])
 @pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
 def test_schedules_equal_the_plain_implementation(folders, name, mode, tmp_path, emu_ops):
     folder = folders[name]
