@@ -5,10 +5,9 @@
 #include "common.h"
 #include <math.h>
 
-// tanh for capped scores, float32: 1 - 2 / (1 + e^2x), the quotient as a product with the hardware's reciprocal (one
-// instruction, an error of one unit in the last place, where the division is a sequence of ten); absolute error of a
-// few 1e-7 (the exponential overflows to the right limit on both sides)
-__device__ __forceinline__ float capped_tanh(float x) { return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __expf(2.0f * x)); }
+// tanh for capped scores, float32: 1 - 2 / (1 + e^2x); absolute error of a few 1e-7 (the exponential overflows to the
+// right limit on both sides)
+__device__ __forceinline__ float capped_tanh(float x) { return 1.0f - 2.0f / (1.0f + __expf(2.0f * x)); }
 
 // Where element (row m, column n) lies when at most 16 * tiles rows are kept in MFMA operand order for a product that
 // reads them next: [n / 32 steps][tiles][64 lanes][8], lane 16 g + m % 16 of tile m / 16 holding columns 32 s + 8 g ...
